@@ -1,0 +1,194 @@
+/*
+ * pplx_a2a.h -- C ABI of the MI355X (gfx950) MoE dispatch / combine library.
+ *
+ * This is the boundary a host-language binding attaches to.  Every entry point
+ * takes plain pointers, sizes and strides; no torch / C++ types cross it.  The
+ * library replaces the host classes and kernels of ppl-ai/pplx-kernels'
+ * intranode all-to-all for a single-GPU loopback: all `world_size` simulated
+ * expert-parallel (EP) ranks live in one process and one GPU's HBM.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   csrc/all_to_all/all_to_all.h:9-13    SplitMode                -> pplx_a2a_split_mode
+ *   csrc/all_to_all/all_to_all.h:29-39   AllToAll ctor arguments  -> pplx_a2a_config_t
+ *   csrc/all_to_all/intranode.h:23-63    AllToAllIntraNode        -> pplx_a2a_t + dispatch/combine
+ *   csrc/core/buffer.h:116-161           Strided1D/2D/3D views    -> pointer + stride fields
+ *   csrc/bindings/all_to_all_ops.cpp:54-108,122-196,238-311  create/destroy/dispatch/combine ops
+ *
+ * Conventions
+ *   - Every function returns a pplx_a2a_status; 0 is success.  The library never
+ *     exits or traps; pplx_a2a_last_error() returns the message of the calling
+ *     thread's last failure.
+ *   - Device pointers are HBM addresses on the world's device.  `stream` is a
+ *     hipStream_t passed as void* (NULL = the legacy default stream).
+ *   - No entry point other than *_create / *_destroy allocates, frees or
+ *     synchronises; dispatch/combine only enqueue kernels, so they may be
+ *     captured in a hipGraph and replayed.
+ */
+#ifndef PPLX_A2A_H_
+#define PPLX_A2A_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum pplx_a2a_status {
+  PPLX_A2A_OK = 0,
+  PPLX_A2A_INVALID_ARGUMENT = 1, /* a precondition on the arguments does not hold */
+  PPLX_A2A_INVALID_STATE = 2,    /* call order violated (e.g. RECV before every SEND) */
+  PPLX_A2A_HIP_ERROR = 3,        /* a HIP runtime call failed */
+  PPLX_A2A_UNSUPPORTED = 4       /* valid request that this build cannot serve */
+} pplx_a2a_status;
+
+/* csrc/all_to_all/all_to_all.h:9-13 */
+typedef enum pplx_a2a_split_mode {
+  PPLX_A2A_SPLIT_NONE = 0, /* send and receive in one call */
+  PPLX_A2A_SPLIT_SEND = 1,
+  PPLX_A2A_SPLIT_RECV = 2
+} pplx_a2a_split_mode;
+
+/* element types of combine: csrc/bindings/all_to_all_ops.cpp:265-310 */
+typedef enum pplx_a2a_dtype {
+  PPLX_A2A_F32 = 0,
+  PPLX_A2A_BF16 = 1,
+  PPLX_A2A_F16 = 2
+} pplx_a2a_dtype;
+
+/* The AllToAll constructor arguments, csrc/all_to_all/all_to_all.h:29-39.
+ * Invariants checked at world creation (csrc/all_to_all/all_to_all.cpp:32-39):
+ * hidden_dim_bytes % 16 == 0, hidden_dim_scale_bytes % 16 == 0,
+ * hidden_dim_scale_bytes <= hidden_dim_bytes, num_experts % world_size == 0,
+ * world_size % dp_size == 0.  Unlike the reference a single DP group
+ * (world_size == dp_size) is accepted. */
+typedef struct pplx_a2a_config {
+  uint64_t max_num_tokens;         /* M: max tokens per DP group per step */
+  uint64_t num_experts;            /* E: global expert count */
+  uint64_t experts_per_token;      /* K: top-k */
+  uint32_t world_size;             /* R: number of simulated EP ranks */
+  uint32_t dp_size;                /* ranks per DP group (hold identical tokens) */
+  uint64_t hidden_dim;             /* H: elements per token row */
+  uint64_t hidden_dim_bytes;       /* bytes of one dispatched activation row */
+  uint64_t hidden_dim_scale_bytes; /* bytes of one row of fp32 block scales, 0 if none */
+} pplx_a2a_config_t;
+
+/* Owner of the state shared by all simulated ranks (routing tables, slot map,
+ * staging for split mode).  Takes the place of the IPC-mapped peer buffers set
+ * up in csrc/all_to_all/intranode.cpp:11-137. */
+typedef struct pplx_a2a_world pplx_a2a_world_t;
+/* One simulated EP rank; takes the place of an AllToAllIntraNode object. */
+typedef struct pplx_a2a pplx_a2a_t;
+/* An instantiated hipGraph. */
+typedef struct pplx_a2a_graph pplx_a2a_graph_t;
+
+/* Arguments of one rank's dispatch: the views built in
+ * csrc/bindings/all_to_all_ops.cpp:165-195 for AllToAllIntraNode::dispatch
+ * (csrc/all_to_all/intranode.h:39-50). */
+typedef struct pplx_a2a_dispatch_args {
+  int32_t *out_expert_num_tokens;        /* [L] */
+  int64_t out_expert_num_tokens_stride;  /* elements */
+  void *out_expert_x;                    /* [L, rows, hidden_dim_bytes] */
+  int64_t out_expert_x_stride_row;       /* bytes between rows */
+  int64_t out_expert_x_stride_expert;    /* bytes between local experts */
+  int64_t out_expert_x_rows;             /* size(1): row capacity per expert; 0 = M * num_dp_groups */
+  float *out_expert_x_scale;             /* [L, rows, S] or NULL */
+  int64_t out_expert_x_scale_stride_elem;   /* floats */
+  int64_t out_expert_x_scale_stride_row;    /* floats */
+  int64_t out_expert_x_scale_stride_expert; /* floats */
+  const void *dp_x;                      /* [m, hidden_dim_bytes] */
+  int64_t dp_x_stride_row;               /* bytes */
+  const float *dp_x_scale;               /* [m, S] or NULL */
+  int64_t dp_x_scale_stride_elem;        /* floats */
+  int64_t dp_x_scale_stride_row;         /* floats */
+  const uint32_t *indices;               /* [m, K] contiguous, distinct experts per row */
+  uint32_t m;                            /* rows of dp_x / indices */
+  const uint32_t *bound_m;               /* device scalar: tokens actually present, or NULL (= m) */
+} pplx_a2a_dispatch_args_t;
+
+/* Arguments of one rank's combine: the views built in
+ * csrc/bindings/all_to_all_ops.cpp:222-235 for AllToAllIntraNode::combine<T,U>
+ * (csrc/all_to_all/intranode.h:53-63).  Strides are in elements. */
+typedef struct pplx_a2a_combine_args {
+  void *out_tokens;                 /* [>= m, H] of out_dtype */
+  int64_t out_tokens_stride_row;
+  int32_t out_dtype;                /* pplx_a2a_dtype: BF16 or F16 */
+  const uint32_t *indices;          /* [m, K] contiguous */
+  const float *weights;             /* [m, K] */
+  int64_t weights_stride_row;
+  const void *expert_y;             /* [L, rows, H] of in_dtype */
+  int64_t expert_y_stride_row;
+  int64_t expert_y_stride_expert;
+  int64_t expert_y_rows;            /* size(1); 0 = M * num_dp_groups */
+  int32_t in_dtype;                 /* pplx_a2a_dtype: F32, BF16 or F16 */
+  uint32_t m;
+  const uint32_t *bound_m;          /* device scalar or NULL (= m) */
+} pplx_a2a_combine_args_t;
+
+/* ---- lifecycle ------------------------------------------------------- */
+
+/* Allocates the world's device state on `device` (a HIP device ordinal).
+ * Replaces the buffer set-up of csrc/all_to_all/intranode.cpp:11-137. */
+int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_world_t **out);
+/* Frees the world.  Fails with INVALID_STATE while rank handles are attached. */
+int pplx_a2a_world_destroy(pplx_a2a_world_t *world);
+
+/* Attaches simulated rank `rank`; replaces create_intranode,
+ * csrc/bindings/all_to_all_ops.cpp:79-106. */
+int pplx_a2a_create(pplx_a2a_world_t *world, uint32_t rank, pplx_a2a_t **out);
+/* Replaces destroy, csrc/bindings/all_to_all_ops.cpp:108. */
+int pplx_a2a_destroy(pplx_a2a_t *handle);
+/* AllToAll::getNumExpertsPerToken, csrc/all_to_all/all_to_all.h:44. */
+uint64_t pplx_a2a_num_experts_per_token(const pplx_a2a_t *handle);
+uint32_t pplx_a2a_rank(const pplx_a2a_t *handle);
+
+/* ---- per-rank calls (the reference API) ------------------------------ */
+
+/* AllToAllIntraNode::dispatch, csrc/all_to_all/intranode_dispatch.cu:288-390.
+ * The call is collective over the world, like the reference's: with
+ * PPLX_A2A_SPLIT_NONE the kernels are enqueued on `stream` when the last of
+ * the world_size ranks has made its call for the step, and every rank's
+ * outputs are complete once they finish.  With SEND / RECV, every rank's SEND
+ * must be enqueued before the first RECV. */
+int pplx_a2a_dispatch(pplx_a2a_t *handle, const pplx_a2a_dispatch_args_t *args,
+                      int split_mode, void *stream);
+/* AllToAllIntraNode::combine<T,U>, csrc/all_to_all/intranode_combine.cu:190-266. */
+int pplx_a2a_combine(pplx_a2a_t *handle, const pplx_a2a_combine_args_t *args,
+                     int split_mode, void *stream);
+
+/* ---- all ranks in one call ------------------------------------------- */
+
+/* One step for all ranks: `per_rank` is a host array of world_size entries,
+ * entry r holding rank r's arguments.  Equivalent to world_size calls of
+ * pplx_a2a_dispatch(..., PPLX_A2A_SPLIT_NONE, stream). */
+int pplx_a2a_world_dispatch(pplx_a2a_world_t *world, const pplx_a2a_dispatch_args_t *per_rank,
+                            void *stream);
+int pplx_a2a_world_combine(pplx_a2a_world_t *world, const pplx_a2a_combine_args_t *per_rank,
+                           void *stream);
+
+/* Reads and clears the world's device-side fault word (synchronises `stream`):
+ * bit 0 = a routed row did not fit out_expert_x_rows and was dropped,
+ * bit 1 = an expert index >= num_experts was ignored,
+ * bit 2 = combine met a slot beyond expert_y_rows. */
+int pplx_a2a_world_faults(pplx_a2a_world_t *world, void *stream, uint32_t *out_bits);
+
+/* ---- hipGraph plumbing ------------------------------------------------ */
+
+/* Thin wrappers over stream capture so that a binding without HIP access can
+ * record a dispatch+combine step once and replay it
+ * (the reference's "CUDA graph support", README.md:5). */
+int pplx_a2a_graph_begin_capture(void *stream);
+int pplx_a2a_graph_end_capture(void *stream, pplx_a2a_graph_t **out);
+int pplx_a2a_graph_launch(pplx_a2a_graph_t *graph, void *stream);
+int pplx_a2a_graph_destroy(pplx_a2a_graph_t *graph);
+
+/* ---- misc -------------------------------------------------------------- */
+
+const char *pplx_a2a_last_error(void);
+/* "major.minor.patch" of this library. */
+const char *pplx_a2a_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PPLX_A2A_H_ */

@@ -1,0 +1,542 @@
+// Host side of the C ABI declared in include/pplx_a2a.h: world / rank-handle
+// lifecycle, argument checks, table binding and kernel sequencing.
+//
+// Takes the place of the reference's host classes
+// (csrc/all_to_all/all_to_all.cpp:8-40, csrc/all_to_all/intranode.cpp:11-162) and
+// of the argument checks in csrc/bindings/all_to_all_ops.cpp:122-196,238-311 that
+// do not depend on torch types.  Failures are reported as status codes plus a
+// thread-local message; nothing here exits or traps.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "a2a_device.h"
+#include "pplx_a2a.h"
+
+using namespace pplx_amd;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int status, const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return status;
+}
+
+#define HIP_TRY(expr)                                                                        \
+  do {                                                                                       \
+    hipError_t err_ = (expr);                                                                \
+    if (err_ != hipSuccess)                                                                  \
+      return fail(PPLX_A2A_HIP_ERROR, "%s failed: %s", #expr, hipGetErrorString(err_));      \
+  } while (0)
+
+#define LAUNCH_TRY(expr)                                                                     \
+  do {                                                                                       \
+    int err_ = (expr);                                                                       \
+    if (err_ != 0)                                                                           \
+      return fail(PPLX_A2A_HIP_ERROR, "%s failed: %s", #expr,                                \
+                  hipGetErrorString((hipError_t)err_));                                      \
+  } while (0)
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Restores the caller's current device on scope exit.
+class DeviceScope {
+ public:
+  explicit DeviceScope(int device) {
+    ok_ = hipGetDevice(&prev_) == hipSuccess;
+    if (ok_ && prev_ != device) ok_ = hipSetDevice(device) == hipSuccess;
+    switched_ = ok_ && prev_ != device;
+  }
+  ~DeviceScope() {
+    if (switched_) (void)hipSetDevice(prev_);
+  }
+  bool ok() const { return ok_; }
+
+ private:
+  int prev_ = 0;
+  bool ok_ = false;
+  bool switched_ = false;
+};
+
+}  // namespace
+
+struct pplx_a2a_world {
+  pplx_a2a_config_t cfg;
+  int device = 0;
+  WorldDev dev{};
+  std::mutex mu;
+  int attached = 0;
+
+  // Arguments recorded for the step being assembled, and which ranks have called.
+  std::vector<DispatchRank> pend_dispatch;
+  std::vector<CombineRank> pend_combine;
+  std::vector<uint8_t> arrived_dispatch, arrived_combine;
+  uint32_t n_arrived_dispatch = 0, n_arrived_combine = 0;
+  int combine_in_dtype = -1, combine_out_dtype = -1;
+
+  // What the device tables currently hold; trusted only while no stream capture
+  // has recorded a bind (a replayed graph rewrites the tables behind our back).
+  std::vector<DispatchRank> bound_dispatch;
+  std::vector<CombineRank> bound_combine;
+  bool bound_dispatch_valid = false, bound_combine_valid = false;
+  bool captured_once = false;
+};
+
+struct pplx_a2a {
+  pplx_a2a_world *world;
+  uint32_t rank;
+};
+
+struct pplx_a2a_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+namespace {
+
+int check_config(const pplx_a2a_config_t &c) {
+  if (c.world_size == 0 || c.dp_size == 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "world_size and dp_size must be positive");
+  if (c.world_size % c.dp_size != 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "world_size must be a multiple of dp_size");
+  if (c.num_experts == 0 || c.num_experts % c.world_size != 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "num_experts must be a positive multiple of world_size");
+  if (c.experts_per_token == 0 || c.experts_per_token > kWave || c.experts_per_token > c.num_experts)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "experts_per_token must be in [1, min(64, num_experts)]");
+  if (c.max_num_tokens == 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "max_num_tokens must be positive");
+  // csrc/all_to_all/all_to_all.cpp:32-39
+  if (c.hidden_dim_bytes == 0 || c.hidden_dim_bytes % 16 != 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "invalid hidden dim bytes");
+  if (c.hidden_dim_scale_bytes % 16 != 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "invalid hidden dim scale bytes");
+  if (c.hidden_dim_scale_bytes > c.hidden_dim_bytes)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "invalid hidden dim bytes");
+  if (c.hidden_dim == 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "hidden_dim must be positive");
+  const uint64_t groups = c.world_size / c.dp_size;
+  if (groups * c.max_num_tokens > (1ull << 30) ||
+      groups * c.max_num_tokens * c.experts_per_token > (1ull << 31) ||
+      c.hidden_dim_bytes > (1ull << 30) || c.num_experts > 5461)
+    return fail(PPLX_A2A_UNSUPPORTED, "geometry exceeds the limits of this build");
+  return PPLX_A2A_OK;
+}
+
+int convert_dispatch(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_dispatch_args_t &a,
+                     DispatchRank *out) {
+  const uint32_t S = w.dev.S;
+  if (!a.out_expert_num_tokens)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_num_tokens is NULL", rank);
+  if (!a.out_expert_x) return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x is NULL", rank);
+  if (a.m > 0 && (!a.dp_x || !a.indices))
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: dp_x / indices is NULL with m > 0", rank);
+  if (S > 0 && !a.out_expert_x_scale)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x_scale is NULL but scales are configured", rank);
+  if (S > 0 && a.m > 0 && !a.dp_x_scale)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: dp_x_scale is NULL but scales are configured", rank);
+  if (!aligned16(a.out_expert_x) || a.out_expert_x_stride_row % 16 || a.out_expert_x_stride_expert % 16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x must be 16-byte aligned with 16-byte strides", rank);
+  if (!aligned16(a.dp_x) || a.dp_x_stride_row % 16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: dp_x must be 16-byte aligned with a 16-byte row stride", rank);
+  if (a.out_expert_x_rows < 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x_rows is negative", rank);
+  const uint64_t rows = a.out_expert_x_rows ? (uint64_t)a.out_expert_x_rows : (uint64_t)w.dev.M * w.dev.G;
+  DispatchRank d{};
+  d.out_num_tokens = a.out_expert_num_tokens;
+  d.out_num_tokens_stride = a.out_expert_num_tokens_stride;
+  d.expert_x = static_cast<uint8_t *>(a.out_expert_x);
+  d.x_stride_row = a.out_expert_x_stride_row;
+  d.x_stride_expert = a.out_expert_x_stride_expert;
+  d.expert_xs = S ? a.out_expert_x_scale : nullptr;
+  d.xs_stride_elem = a.out_expert_x_scale_stride_elem;
+  d.xs_stride_row = a.out_expert_x_scale_stride_row;
+  d.xs_stride_expert = a.out_expert_x_scale_stride_expert;
+  d.dp_x = static_cast<const uint8_t *>(a.dp_x);
+  d.dp_x_stride_row = a.dp_x_stride_row;
+  d.dp_xs = S ? a.dp_x_scale : nullptr;
+  d.dp_xs_stride_elem = a.dp_x_scale_stride_elem;
+  d.dp_xs_stride_row = a.dp_x_scale_stride_row;
+  d.indices = a.indices;
+  d.bound_m = a.bound_m;
+  d.m = a.m;
+  d.x_rows = rows > 0xfffffffeull ? 0xfffffffeu : (uint32_t)rows;
+  *out = d;
+  return PPLX_A2A_OK;
+}
+
+size_t dtype_size(int dt) { return dt == PPLX_A2A_F32 ? 4 : 2; }
+
+int convert_combine(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_combine_args_t &a,
+                    CombineRank *out) {
+  // csrc/bindings/all_to_all_ops.cpp:265-310
+  if (a.in_dtype != PPLX_A2A_F32 && a.in_dtype != PPLX_A2A_BF16 && a.in_dtype != PPLX_A2A_F16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "Unsupported dtype for expertY");
+  if (a.out_dtype != PPLX_A2A_BF16 && a.out_dtype != PPLX_A2A_F16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "Unsupported dtype for outTokens");
+  if (w.dev.H % 8 != 0)
+    return fail(PPLX_A2A_UNSUPPORTED, "combine needs hidden_dim to be a multiple of 8");
+  if (!a.expert_y) return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y is NULL", rank);
+  if (a.m > 0 && (!a.out_tokens || !a.indices || !a.weights))
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_tokens / indices / weights is NULL with m > 0", rank);
+  const size_t in_sz = dtype_size(a.in_dtype), out_sz = dtype_size(a.out_dtype);
+  if (!aligned16(a.expert_y) || (a.expert_y_stride_row * (int64_t)in_sz) % 16 ||
+      (a.expert_y_stride_expert * (int64_t)in_sz) % 16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y must be 16-byte aligned with 16-byte strides", rank);
+  if (!aligned16(a.out_tokens) || (a.out_tokens_stride_row * (int64_t)out_sz) % 16)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_tokens must be 16-byte aligned with a 16-byte row stride", rank);
+  if (a.expert_y_rows < 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y_rows is negative", rank);
+  const uint64_t rows = a.expert_y_rows ? (uint64_t)a.expert_y_rows : (uint64_t)w.dev.M * w.dev.G;
+  CombineRank c{};
+  c.out_tokens = a.out_tokens;
+  c.out_stride_row = a.out_tokens_stride_row;
+  c.indices = a.indices;
+  c.weights = a.weights;
+  c.w_stride_row = a.weights_stride_row;
+  c.expert_y = a.expert_y;
+  c.y_stride_row = a.expert_y_stride_row;
+  c.y_stride_expert = a.expert_y_stride_expert;
+  c.bound_m = a.bound_m;
+  c.m = a.m;
+  c.y_rows = rows > 0xfffffffeull ? 0xfffffffeu : (uint32_t)rows;
+  *out = c;
+  return PPLX_A2A_OK;
+}
+
+int stream_is_capturing(void *stream, bool *out) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &st));
+  *out = st != hipStreamCaptureStatusNone;
+  return PPLX_A2A_OK;
+}
+
+// Makes the device tables equal to `rows`, batch by batch, skipping batches the
+// tables are known to hold already.
+template <typename Row, typename Batch, typename Launch>
+int flush_table(pplx_a2a_world &w, const std::vector<Row> &rows, std::vector<Row> &bound,
+                bool &bound_valid, bool force, Launch launch, void *stream) {
+  const uint32_t R = w.dev.R;
+  for (uint32_t first = 0; first < R; first += kBindBatch) {
+    const uint32_t count = (R - first < kBindBatch) ? R - first : kBindBatch;
+    bool dirty = force || !bound_valid;
+    if (!dirty) dirty = memcmp(&rows[first], &bound[first], sizeof(Row) * count) != 0;
+    if (!dirty) continue;
+    Batch b;
+    memset(static_cast<void *>(&b), 0, sizeof(b));
+    b.first = first;
+    b.count = count;
+    memcpy(static_cast<void *>(b.rows), &rows[first], sizeof(Row) * count);
+    LAUNCH_TRY(launch(w.dev, b, stream));
+  }
+  bound = rows;
+  bound_valid = true;
+  return PPLX_A2A_OK;
+}
+
+int run_dispatch(pplx_a2a_world &w, void *stream) {
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  bool capturing = false;
+  int st = stream_is_capturing(stream, &capturing);
+  if (st) return st;
+  if (capturing) w.captured_once = true;
+  st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
+                                                    w.bound_dispatch_valid, w.captured_once,
+                                                    launch_bind_dispatch, stream);
+  if (st) return st;
+  LAUNCH_TRY(launch_route(w.dev, stream));
+  LAUNCH_TRY(launch_dispatch_scatter(w.dev, stream));
+  return PPLX_A2A_OK;
+}
+
+int run_combine(pplx_a2a_world &w, void *stream) {
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  bool capturing = false;
+  int st = stream_is_capturing(stream, &capturing);
+  if (st) return st;
+  if (capturing) w.captured_once = true;
+  st = flush_table<CombineRank, BindCombineBatch>(w, w.pend_combine, w.bound_combine,
+                                                  w.bound_combine_valid, w.captured_once,
+                                                  launch_bind_combine, stream);
+  if (st) return st;
+  LAUNCH_TRY(launch_combine_gather(w.dev, w.combine_in_dtype, w.combine_out_dtype, stream));
+  return PPLX_A2A_OK;
+}
+
+void reset_dispatch_arrivals(pplx_a2a_world &w) {
+  std::fill(w.arrived_dispatch.begin(), w.arrived_dispatch.end(), 0);
+  w.n_arrived_dispatch = 0;
+}
+
+void reset_combine_arrivals(pplx_a2a_world &w) {
+  std::fill(w.arrived_combine.begin(), w.arrived_combine.end(), 0);
+  w.n_arrived_combine = 0;
+  w.combine_in_dtype = w.combine_out_dtype = -1;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *pplx_a2a_last_error(void) { return g_last_error.c_str(); }
+
+const char *pplx_a2a_version(void) { return "0.1.0"; }
+
+int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_world_t **out) {
+  if (!cfg || !out) return fail(PPLX_A2A_INVALID_ARGUMENT, "cfg / out is NULL");
+  *out = nullptr;
+  int st = check_config(*cfg);
+  if (st) return st;
+  int n_dev = 0;
+  HIP_TRY(hipGetDeviceCount(&n_dev));
+  if (device < 0 || device >= n_dev)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "device %d out of range (%d visible)", device, n_dev);
+  DeviceScope scope(device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", device);
+
+  pplx_a2a_world *w = new (std::nothrow) pplx_a2a_world();
+  if (!w) return fail(PPLX_A2A_HIP_ERROR, "out of host memory");
+  w->cfg = *cfg;
+  w->device = device;
+  WorldDev &d = w->dev;
+  d.R = cfg->world_size;
+  d.dp = cfg->dp_size;
+  d.G = d.R / d.dp;
+  d.M = (uint32_t)cfg->max_num_tokens;
+  d.E = (uint32_t)cfg->num_experts;
+  d.L = d.E / d.R;
+  d.K = (uint32_t)cfg->experts_per_token;
+  d.H = (uint32_t)cfg->hidden_dim;
+  d.Hb = (uint32_t)cfg->hidden_dim_bytes;
+  d.S = (uint32_t)(cfg->hidden_dim_scale_bytes / 4);
+  // Largest power-of-two chunk count (<= 16) whose LDS tables fit 64 KiB.
+  d.tile_chunks = 16;
+  while (d.tile_chunks > 1 && route_lds_bytes(d.E, d.tile_chunks) > 65536u) d.tile_chunks /= 2;
+  const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
+  d.num_tiles = (uint32_t)(((uint64_t)d.G * d.M + tile_tokens - 1) / tile_tokens);
+
+  auto cleanup = [&]() {
+    (void)hipFree(d.drank);
+    (void)hipFree(d.crank);
+    (void)hipFree(d.tile_cnt);
+    (void)hipFree(d.slot_map);
+    (void)hipFree(d.faults);
+    delete w;
+  };
+  struct Alloc {
+    void **ptr;
+    size_t bytes;
+  } allocs[] = {
+      {reinterpret_cast<void **>(&d.drank), sizeof(DispatchRank) * d.R},
+      {reinterpret_cast<void **>(&d.crank), sizeof(CombineRank) * d.R},
+      {reinterpret_cast<void **>(&d.tile_cnt), sizeof(uint32_t) * (size_t)d.num_tiles * d.E},
+      {reinterpret_cast<void **>(&d.slot_map), sizeof(uint32_t) * (size_t)d.G * d.M * d.K},
+      {reinterpret_cast<void **>(&d.faults), 256},
+  };
+  for (const Alloc &a : allocs) {
+    hipError_t err = hipMalloc(a.ptr, a.bytes);
+    if (err == hipSuccess) err = hipMemset(*a.ptr, 0, a.bytes);
+    if (err != hipSuccess) {
+      cleanup();
+      return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of world state failed: %s", a.bytes,
+                  hipGetErrorString(err));
+    }
+  }
+  w->pend_dispatch.assign(d.R, DispatchRank{});
+  w->pend_combine.assign(d.R, CombineRank{});
+  w->bound_dispatch.assign(d.R, DispatchRank{});
+  w->bound_combine.assign(d.R, CombineRank{});
+  w->arrived_dispatch.assign(d.R, 0);
+  w->arrived_combine.assign(d.R, 0);
+  *out = w;
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_world_destroy(pplx_a2a_world_t *w) {
+  if (!w) return PPLX_A2A_OK;
+  if (w->attached != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "%d rank handle(s) still attached to the world", w->attached);
+  DeviceScope scope(w->device);
+  (void)hipDeviceSynchronize();
+  (void)hipFree(w->dev.drank);
+  (void)hipFree(w->dev.crank);
+  (void)hipFree(w->dev.tile_cnt);
+  (void)hipFree(w->dev.slot_map);
+  (void)hipFree(w->dev.faults);
+  delete w;
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_create(pplx_a2a_world_t *w, uint32_t rank, pplx_a2a_t **out) {
+  if (!w || !out) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / out is NULL");
+  *out = nullptr;
+  if (rank >= w->dev.R)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u out of range for world_size %u", rank, w->dev.R);
+  pplx_a2a *h = new (std::nothrow) pplx_a2a{w, rank};
+  if (!h) return fail(PPLX_A2A_HIP_ERROR, "out of host memory");
+  std::lock_guard<std::mutex> lock(w->mu);
+  ++w->attached;
+  *out = h;
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_destroy(pplx_a2a_t *h) {
+  if (!h) return PPLX_A2A_OK;
+  {
+    std::lock_guard<std::mutex> lock(h->world->mu);
+    --h->world->attached;
+  }
+  delete h;
+  return PPLX_A2A_OK;
+}
+
+uint64_t pplx_a2a_num_experts_per_token(const pplx_a2a_t *h) { return h ? h->world->dev.K : 0; }
+
+uint32_t pplx_a2a_rank(const pplx_a2a_t *h) { return h ? h->rank : 0; }
+
+int pplx_a2a_dispatch(pplx_a2a_t *h, const pplx_a2a_dispatch_args_t *args, int split_mode,
+                      void *stream) {
+  if (!h || !args) return fail(PPLX_A2A_INVALID_ARGUMENT, "handle / args is NULL");
+  pplx_a2a_world &w = *h->world;
+  if (split_mode != PPLX_A2A_SPLIT_NONE && split_mode != PPLX_A2A_SPLIT_SEND &&
+      split_mode != PPLX_A2A_SPLIT_RECV)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
+  if (split_mode != PPLX_A2A_SPLIT_NONE)
+    return fail(PPLX_A2A_UNSUPPORTED, "split send/recv dispatch is not available in this build");
+  DispatchRank row;
+  int st = convert_dispatch(w, h->rank, *args, &row);
+  if (st) return st;
+  std::lock_guard<std::mutex> lock(w.mu);
+  if (w.arrived_dispatch[h->rank])
+    return fail(PPLX_A2A_INVALID_STATE,
+                "rank %u called dispatch twice before the other ranks of the step", h->rank);
+  w.pend_dispatch[h->rank] = row;
+  w.arrived_dispatch[h->rank] = 1;
+  if (++w.n_arrived_dispatch < w.dev.R) return PPLX_A2A_OK;
+  reset_dispatch_arrivals(w);
+  return run_dispatch(w, stream);
+}
+
+int pplx_a2a_combine(pplx_a2a_t *h, const pplx_a2a_combine_args_t *args, int split_mode,
+                     void *stream) {
+  if (!h || !args) return fail(PPLX_A2A_INVALID_ARGUMENT, "handle / args is NULL");
+  pplx_a2a_world &w = *h->world;
+  if (split_mode != PPLX_A2A_SPLIT_NONE && split_mode != PPLX_A2A_SPLIT_SEND &&
+      split_mode != PPLX_A2A_SPLIT_RECV)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
+  if (split_mode != PPLX_A2A_SPLIT_NONE)
+    return fail(PPLX_A2A_UNSUPPORTED, "split send/recv combine is not available in this build");
+  CombineRank row;
+  int st = convert_combine(w, h->rank, *args, &row);
+  if (st) return st;
+  std::lock_guard<std::mutex> lock(w.mu);
+  if (w.arrived_combine[h->rank])
+    return fail(PPLX_A2A_INVALID_STATE,
+                "rank %u called combine twice before the other ranks of the step", h->rank);
+  if (w.n_arrived_combine > 0 &&
+      (w.combine_in_dtype != args->in_dtype || w.combine_out_dtype != args->out_dtype))
+    return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
+  w.combine_in_dtype = args->in_dtype;
+  w.combine_out_dtype = args->out_dtype;
+  w.pend_combine[h->rank] = row;
+  w.arrived_combine[h->rank] = 1;
+  if (++w.n_arrived_combine < w.dev.R) return PPLX_A2A_OK;
+  const int in_dt = w.combine_in_dtype, out_dt = w.combine_out_dtype;
+  reset_combine_arrivals(w);
+  w.combine_in_dtype = in_dt;
+  w.combine_out_dtype = out_dt;
+  return run_combine(w, stream);
+}
+
+int pplx_a2a_world_dispatch(pplx_a2a_world_t *w, const pplx_a2a_dispatch_args_t *per_rank,
+                            void *stream) {
+  if (!w || !per_rank) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / per_rank is NULL");
+  std::lock_guard<std::mutex> lock(w->mu);
+  if (w->n_arrived_dispatch != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a per-rank dispatch step is still being assembled");
+  for (uint32_t r = 0; r < w->dev.R; ++r) {
+    int st = convert_dispatch(*w, r, per_rank[r], &w->pend_dispatch[r]);
+    if (st) return st;
+  }
+  return run_dispatch(*w, stream);
+}
+
+int pplx_a2a_world_combine(pplx_a2a_world_t *w, const pplx_a2a_combine_args_t *per_rank,
+                           void *stream) {
+  if (!w || !per_rank) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / per_rank is NULL");
+  std::lock_guard<std::mutex> lock(w->mu);
+  if (w->n_arrived_combine != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a per-rank combine step is still being assembled");
+  for (uint32_t r = 0; r < w->dev.R; ++r) {
+    if (per_rank[r].in_dtype != per_rank[0].in_dtype || per_rank[r].out_dtype != per_rank[0].out_dtype)
+      return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
+    int st = convert_combine(*w, r, per_rank[r], &w->pend_combine[r]);
+    if (st) return st;
+  }
+  w->combine_in_dtype = per_rank[0].in_dtype;
+  w->combine_out_dtype = per_rank[0].out_dtype;
+  return run_combine(*w, stream);
+}
+
+int pplx_a2a_world_faults(pplx_a2a_world_t *w, void *stream, uint32_t *out_bits) {
+  if (!w || !out_bits) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / out_bits is NULL");
+  DeviceScope scope(w->device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w->device);
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  uint32_t bits = 0;
+  HIP_TRY(hipMemcpy(&bits, w->dev.faults, sizeof(bits), hipMemcpyDeviceToHost));
+  if (bits) HIP_TRY(hipMemset(w->dev.faults, 0, sizeof(bits)));
+  *out_bits = bits;
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_graph_begin_capture(void *stream) {
+  HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_graph_end_capture(void *stream, pplx_a2a_graph_t **out) {
+  if (!out) return fail(PPLX_A2A_INVALID_ARGUMENT, "out is NULL");
+  *out = nullptr;
+  pplx_a2a_graph *g = new (std::nothrow) pplx_a2a_graph();
+  if (!g) return fail(PPLX_A2A_HIP_ERROR, "out of host memory");
+  hipError_t err = hipStreamEndCapture((hipStream_t)stream, &g->graph);
+  if (err == hipSuccess) err = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+  if (err != hipSuccess) {
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+    return fail(PPLX_A2A_HIP_ERROR, "graph capture failed: %s", hipGetErrorString(err));
+  }
+  *out = g;
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_graph_launch(pplx_a2a_graph_t *g, void *stream) {
+  if (!g) return fail(PPLX_A2A_INVALID_ARGUMENT, "graph is NULL");
+  HIP_TRY(hipGraphLaunch(g->exec, (hipStream_t)stream));
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_graph_destroy(pplx_a2a_graph_t *g) {
+  if (!g) return PPLX_A2A_OK;
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  if (g->graph) (void)hipGraphDestroy(g->graph);
+  delete g;
+  return PPLX_A2A_OK;
+}
+
+}  // extern "C"

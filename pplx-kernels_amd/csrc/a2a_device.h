@@ -1,0 +1,102 @@
+// Device-visible records shared by the host layer and the kernels.
+//
+// One DispatchRank / CombineRank row per simulated EP rank lives in a table in
+// HBM; kernels index it by rank.  They carry what the reference passes as
+// Strided1D/2D/3D views (csrc/core/buffer.h:116-161) in the kernel argument
+// lists of csrc/all_to_all/intranode_dispatch.cu:15-53 and
+// csrc/all_to_all/intranode_combine.cu:16-47.
+#pragma once
+
+#include <cstdint>
+
+namespace pplx_amd {
+
+constexpr uint32_t kWave = 64;            // gfx950 wavefront
+constexpr uint32_t kInvalidSlot = 0xffffffffu;
+
+constexpr uint32_t kFaultRowDropped = 1u;   // slot >= out_expert_x rows
+constexpr uint32_t kFaultBadExpert = 2u;    // index >= num_experts
+constexpr uint32_t kFaultBadSlot = 4u;      // combine slot >= expert_y rows
+
+struct alignas(16) DispatchRank {
+  int32_t *out_num_tokens;
+  int64_t out_num_tokens_stride;
+  uint8_t *expert_x;
+  int64_t x_stride_row;     // bytes
+  int64_t x_stride_expert;  // bytes
+  float *expert_xs;
+  int64_t xs_stride_elem;   // floats
+  int64_t xs_stride_row;
+  int64_t xs_stride_expert;
+  const uint8_t *dp_x;
+  int64_t dp_x_stride_row;  // bytes
+  const float *dp_xs;
+  int64_t dp_xs_stride_elem;
+  int64_t dp_xs_stride_row;
+  const uint32_t *indices;
+  const uint32_t *bound_m;
+  uint32_t m;
+  uint32_t x_rows;
+  uint64_t pad_;
+};
+static_assert(sizeof(DispatchRank) == 144, "DispatchRank layout");
+
+struct alignas(16) CombineRank {
+  void *out_tokens;
+  int64_t out_stride_row;   // elements
+  const uint32_t *indices;
+  const float *weights;
+  int64_t w_stride_row;
+  const void *expert_y;
+  int64_t y_stride_row;     // elements
+  int64_t y_stride_expert;
+  const uint32_t *bound_m;
+  uint32_t m;
+  uint32_t y_rows;
+};
+static_assert(sizeof(CombineRank) == 80, "CombineRank layout");
+
+// Geometry + scratch of a world; passed to every kernel by value.
+struct WorldDev {
+  uint32_t R;        // simulated ranks
+  uint32_t dp;       // ranks per DP group
+  uint32_t G;        // DP groups = R / dp
+  uint32_t M;        // max tokens per DP group
+  uint32_t E;        // experts
+  uint32_t L;        // experts per rank
+  uint32_t K;        // experts per token
+  uint32_t H;        // elements per row
+  uint32_t Hb;       // bytes per dispatched row
+  uint32_t S;        // fp32 scales per row
+  uint32_t tile_chunks;  // 64-token chunks per routing tile
+  uint32_t num_tiles;    // ceil(G * M / (64 * tile_chunks))
+  DispatchRank *drank;   // [R]
+  CombineRank *crank;    // [R]
+  uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile
+  uint32_t *slot_map;    // [G * M][K] row of (token, pick) inside its expert
+  uint32_t *faults;      // [1] sticky fault bits
+};
+
+// Up to kBindBatch table rows travel as kernel arguments of one bind launch.
+constexpr uint32_t kBindBatch = 16;
+struct BindDispatchBatch {
+  uint32_t first, count;
+  uint64_t pad_;
+  DispatchRank rows[kBindBatch];
+};
+struct BindCombineBatch {
+  uint32_t first, count;
+  uint64_t pad_;
+  CombineRank rows[kBindBatch];
+};
+
+// Launchers implemented in a2a_kernels.hip; return a hipError_t as int.
+int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream);
+int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stream);
+int launch_route(const WorldDev &w, void *stream);
+int launch_dispatch_scatter(const WorldDev &w, void *stream);
+int launch_combine_gather(const WorldDev &w, int in_dtype, int out_dtype, void *stream);
+// LDS bytes the routing kernels need for a given geometry.
+uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks);
+
+}  // namespace pplx_amd
