@@ -1,0 +1,302 @@
+"""Benchmark of the MoE dispatch + combine hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--all]
+
+A *step* is one dispatch + one combine over all simulated ranks of the workload, replayed
+from a captured hipGraph (inputs resident in HBM).  To keep the working set from living in
+the 256 MB last-level cache between steps, the steps rotate over several independent buffer
+sets, so every timed step touches memory that was last used several steps ago.
+
+Prints ONE JSON line.  ``value`` is the mean step latency in microseconds on the workload
+the metric is quoted on (C2: DeepSeek-V3 shape, 128 tokens/rank, 8 simulated ranks).
+``roofline`` is for the dominant kernel (``combine_gather``): algorithmic bytes per launch
+divided by its mean duration, measured with HIP events around graph replays that contain
+only launches of that kernel.  ``cpu_baseline`` times the oracle's vectorised torch CPU port
+of the same step on this host's cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "pplx-kernels_amd"), ROOT):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+LLC_BYTES = 256 << 20
+
+
+def build_steps(spec, groups, cap, n_sets):
+    from tests.all_to_all_utils import DeviceStep
+
+    steps = []
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    for _ in range(n_sets):
+        st = DeviceStep(spec, groups, cap=cap)
+        # N(0,1) expert outputs in the rows that will be read; fill in slabs to bound memory
+        for r in range(spec.world_size):
+            st.expert_y_all[r].copy_(
+                torch.randn(st.expert_y_all[r].shape, generator=gen, device="cuda", dtype=torch.bfloat16)
+            )
+        steps.append(st)
+    return steps
+
+
+def time_graphs(graphs, order, stream, warmup, repeats=1):
+    """Mean microseconds per graph launch over `order` (a list of graph indices), HIP events
+    on the launch stream."""
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            graphs[order[i % len(order)]].replay(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        start.record(stream)
+        for _ in range(repeats):
+            for i in order:
+                graphs[i].replay(stream)
+        end.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+    return start.elapsed_time(end) * 1e3 / (len(order) * repeats)
+
+
+def capture(world, stream, body):
+    with torch.cuda.stream(stream):
+        body()  # eager once: binds tables, warms code objects
+        stream.synchronize()
+        with world.capture() as cap:
+            body()
+    return cap.graph
+
+
+def measure_workload(name, spec, steps_k, warmup, detail=True):
+    from tests.all_to_all_utils import expert_counts, generate, make_world
+
+    groups = generate(spec)
+    counts = expert_counts(groups, spec.num_experts)
+    cap = max(int(counts.max()), 1)
+    full_cap = spec.max_num_tokens * spec.num_dp_groups
+    if spec.num_experts * full_cap * spec.hidden_dim * 3 < (8 << 30):
+        cap = full_cap  # small enough: use the reference's own sizing
+    disp_b, comb_b = None, None
+    # enough buffer sets that a step's data is evicted before it is used again
+    probe_bytes = sum(g.n for g in groups) * spec.experts_per_token * spec.hidden_dim * 3
+    n_sets = max(2, min(8, int(2.5 * LLC_BYTES / max(probe_bytes, 1)) + 1))
+    per_set = spec.num_experts * cap * spec.hidden_dim * (spec.in_dtype.itemsize + 2)
+    n_sets = max(1, min(n_sets, int((160 << 30) // max(per_set, 1))))
+    steps = build_steps(spec, groups, cap, n_sets)
+    disp_b, comb_b = steps[0].algorithmic_bytes()
+    world = make_world(spec, group_name=f"bench-{name}")
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+
+    def both(st):
+        return lambda: (st.dispatch_world(world), st.combine_world(world))
+
+    step_graphs = [capture(world, stream, both(st)) for st in steps]
+    order = [i % n_sets for i in range(steps_k)]
+    step_us = time_graphs(step_graphs, order, stream, warmup)
+
+    out = {
+        "workload": spec.name,
+        "tokens": int(sum(g.n for g in groups)),
+        "pairs": int(sum(g.n for g in groups) * spec.experts_per_token),
+        "rows_per_expert_capacity": cap,
+        "buffer_sets": n_sets,
+        "dispatch_bytes": disp_b,
+        "combine_bytes": comb_b,
+        "step_us": step_us,
+        "step_GBps": (disp_b + comb_b) / step_us / 1e3,
+        "step_hbm_frac": (disp_b + comb_b) / step_us / 1e3 / HBM_PEAK_GBPS,
+    }
+    if detail:
+        d_graphs = [capture(world, stream, lambda st=st: st.dispatch_world(world)) for st in steps]
+        c_graphs = [capture(world, stream, lambda st=st: st.combine_world(world)) for st in steps]
+        reps = max(1, steps_k // n_sets)
+        d_us = time_graphs(d_graphs, list(range(n_sets)), stream, warmup, reps)
+        c_us = time_graphs(c_graphs, list(range(n_sets)), stream, warmup, reps)
+        # eager (host-launched) step for comparison
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                both(steps[0])()
+            stream.synchronize()
+            t0 = time.perf_counter()
+            for i in range(min(steps_k, 50)):
+                both(steps[i % n_sets])()
+            stream.synchronize()
+            eager_us = (time.perf_counter() - t0) * 1e6 / min(steps_k, 50)
+        out.update(
+            dispatch_us=d_us,
+            combine_us=c_us,
+            dispatch_GBps=disp_b / d_us / 1e3,
+            combine_GBps=comb_b / c_us / 1e3,
+            dispatch_hbm_frac=disp_b / d_us / 1e3 / HBM_PEAK_GBPS,
+            combine_hbm_frac=comb_b / c_us / 1e3 / HBM_PEAK_GBPS,
+            eager_step_us=eager_us,
+        )
+        for g in d_graphs + c_graphs:
+            g.destroy()
+    for g in step_graphs:
+        g.destroy()
+    assert world.faults() == 0, "device-side fault bits set during the benchmark"
+    world.destroy()
+    return out, groups, steps
+
+
+def cpu_baseline(spec, groups, budget_s=20.0):
+    """The oracle's vectorised torch CPU port of one full step, on all host cores."""
+    from oracle import a2a_oracle as orc
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    M, E, K, H = spec.max_num_tokens, spec.num_experts, spec.experts_per_token, spec.hidden_dim
+    cap = M * spec.num_dp_groups
+    groups_t = [(g.x, g.x_scale, g.indices.to(torch.int64), g.n) for g in groups]
+    weights_t = [g.weights for g in groups]
+    # N(0,1) rows; one [cap, H] slab replicated per expert keeps the set-up short
+    slab = torch.randn(cap, H, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    expert_y = slab.unsqueeze(0).expand(E, cap, H).contiguous()
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_all < budget_s / 2 and len(times) < 15):
+        t0 = time.perf_counter()
+        _, _, _, slot_flat = orc.torch_dispatch(groups_t, M, E, K, cap)
+        orc.torch_combine(groups_t, weights_t, slot_flat, expert_y, torch.bfloat16)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > budget_s:
+            break
+    return {
+        "value": statistics.median(times) * 1e6,
+        "unit": "us",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{len(times)} full steps of the same workload (all {sum(g.n for g in groups)} tokens), "
+        "median; torch CPU stable-argsort scatter + fp32 gather-sum (oracle.a2a_oracle.torch_*)",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2")
+    ap.add_argument("--all", action="store_true", help="also measure C1, C3, C4, C5 (reported under 'other_workloads')")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(
+            "bench.py: this build is a single-GPU loopback (all simulated EP ranks share one HBM); "
+            "run it with --gpus 1",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    from pplx_kernels import ops
+    from tests.all_to_all_utils import baseline_configs
+
+    ops.load_library()  # fail loudly here if the HIP library is missing
+    specs = baseline_configs()
+    spec = specs[args.workload]
+    main_res, groups, steps = measure_workload(args.workload, spec, args.steps, args.warmup)
+
+    # Roofline of the dominant kernel: graphs holding back-to-back combine_gather launches
+    # only (the table bind is recorded once per graph), rotating buffer sets.
+    from tests.all_to_all_utils import make_world
+
+    world = make_world(spec, group_name="bench-roofline")
+    stream = torch.cuda.Stream()
+    n_sets = len(steps)
+    launches_per_graph = 8
+
+    def many_combines(st):
+        def body():
+            for _ in range(launches_per_graph):
+                st.combine_world(world)
+        return body
+
+    with torch.cuda.stream(stream):
+        for st in steps:
+            st.dispatch_world(world)  # slot map of this world
+        stream.synchronize()
+    # combine reads the world's slot map, identical for every buffer set (same routing)
+    k_graphs = [capture(world, stream, many_combines(st)) for st in steps]
+    reps = max(1, args.steps // (n_sets * launches_per_graph))
+    per_graph_us = time_graphs(k_graphs, list(range(n_sets)), stream, 2, reps)
+    kernel_us = per_graph_us / launches_per_graph
+    for g in k_graphs:
+        g.destroy()
+    world.destroy()
+    comb_b = main_res["combine_bytes"]
+    roofline = {
+        "kernel": "combine_gather<bf16,bf16>",
+        "bound": "hbm",
+        "achieved": comb_b / kernel_us / 1e3,
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": comb_b / kernel_us / 1e3 / HBM_PEAK_GBPS,
+        "traffic": None,
+        "bytes_per_launch": comb_b,
+        "avg_launch_us": kernel_us,
+        "launches_timed": reps * n_sets * launches_per_graph,
+    }
+
+    result = {
+        "metric": "dispatch+combine latency (us) and achieved HBM GB/s, DSv3 shape 128 tok/rank, 1 GPU",
+        "value": main_res["step_us"],
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["step_us"] / 1e3,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": spec.name,
+            "simulated_ranks": spec.world_size,
+            "num_experts": spec.num_experts,
+            "experts_per_token": spec.experts_per_token,
+            "hidden_dim": spec.hidden_dim,
+            "tokens_per_rank": spec.max_num_tokens,
+            "in_dtype": str(spec.in_dtype).replace("torch.", ""),
+            "out_dtype": str(spec.out_dtype).replace("torch.", ""),
+            "timed": "hipGraph replay of dispatch+combine, rotating buffer sets",
+        },
+        "roofline": roofline,
+        "detail": main_res,
+    }
+    if not args.no_cpu:
+        del steps
+        torch.cuda.empty_cache()
+        result["cpu_baseline"] = cpu_baseline(spec, groups)
+    if args.all:
+        others = {}
+        for name, sp in specs.items():
+            if name == args.workload:
+                continue
+            k = args.steps if name != "C5" else max(8, args.steps // 10)
+            others[name], _, st = measure_workload(name, sp, k, min(args.warmup, 5))
+            del st
+            torch.cuda.empty_cache()
+        result["other_workloads"] = others
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -93,6 +93,8 @@ struct pplx_a2a_world {
   std::vector<CombineRank> bound_combine;
   bool bound_dispatch_valid = false, bound_combine_valid = false;
   bool captured_once = false;
+  // Capture session that recorded the last bind of each table (0 = an eager bind).
+  unsigned long long bind_capture_dispatch = 0, bind_capture_combine = 0;
 };
 
 struct pplx_a2a {
@@ -216,11 +218,27 @@ int convert_combine(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_combi
   return PPLX_A2A_OK;
 }
 
-int stream_is_capturing(void *stream, bool *out) {
+// Capture session of `stream` (0 when it is not capturing).
+int capture_session(void *stream, unsigned long long *out) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-  HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &st));
-  *out = st != hipStreamCaptureStatusNone;
+  unsigned long long id = 0;
+  HIP_TRY(hipStreamGetCaptureInfo((hipStream_t)stream, &st, &id));
+  *out = st == hipStreamCaptureStatusNone ? 0ull : (id ? id : ~0ull);
   return PPLX_A2A_OK;
+}
+
+// Decides whether the host mirror of a device table may be trusted for this call.
+// Inside a capture only binds recorded earlier in the same capture count; in eager
+// mode the mirror is void once any graph exists, because a replay rewrites the table.
+void settle_mirror(pplx_a2a_world &w, unsigned long long session, unsigned long long &last_session,
+                   bool &bound_valid) {
+  if (session != 0) {
+    w.captured_once = true;
+    if (last_session != session) bound_valid = false;
+  } else if (w.captured_once) {
+    bound_valid = false;
+  }
+  last_session = session;
 }
 
 // Makes the device tables equal to `rows`, batch by batch, skipping batches the
@@ -249,31 +267,39 @@ int flush_table(pplx_a2a_world &w, const std::vector<Row> &rows, std::vector<Row
 int run_dispatch(pplx_a2a_world &w, void *stream) {
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
-  bool capturing = false;
-  int st = stream_is_capturing(stream, &capturing);
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
   if (st) return st;
-  if (capturing) w.captured_once = true;
+  settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
+  if (w.dev.R <= kInlineRanks) {
+    LAUNCH_TRY(launch_dispatch(w.dev, w.pend_dispatch.data(), stream));
+    return PPLX_A2A_OK;
+  }
   st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
-                                                    w.bound_dispatch_valid, w.captured_once,
+                                                    w.bound_dispatch_valid, false,
                                                     launch_bind_dispatch, stream);
   if (st) return st;
-  LAUNCH_TRY(launch_route(w.dev, stream));
-  LAUNCH_TRY(launch_dispatch_scatter(w.dev, stream));
+  LAUNCH_TRY(launch_dispatch(w.dev, nullptr, stream));
   return PPLX_A2A_OK;
 }
 
 int run_combine(pplx_a2a_world &w, void *stream) {
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
-  bool capturing = false;
-  int st = stream_is_capturing(stream, &capturing);
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
   if (st) return st;
-  if (capturing) w.captured_once = true;
+  settle_mirror(w, session, w.bind_capture_combine, w.bound_combine_valid);
+  if (w.dev.R <= kInlineRanks) {
+    LAUNCH_TRY(launch_combine(w.dev, w.pend_combine.data(), w.combine_in_dtype, w.combine_out_dtype,
+                              stream));
+    return PPLX_A2A_OK;
+  }
   st = flush_table<CombineRank, BindCombineBatch>(w, w.pend_combine, w.bound_combine,
-                                                  w.bound_combine_valid, w.captured_once,
+                                                  w.bound_combine_valid, false,
                                                   launch_bind_combine, stream);
   if (st) return st;
-  LAUNCH_TRY(launch_combine_gather(w.dev, w.combine_in_dtype, w.combine_out_dtype, stream));
+  LAUNCH_TRY(launch_combine(w.dev, nullptr, w.combine_in_dtype, w.combine_out_dtype, stream));
   return PPLX_A2A_OK;
 }
 

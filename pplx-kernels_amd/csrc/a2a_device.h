@@ -77,8 +77,14 @@ struct WorldDev {
   uint32_t *faults;      // [1] sticky fault bits
 };
 
-// Up to kBindBatch table rows travel as kernel arguments of one bind launch.
+// Worlds of up to kInlineRanks ranks pass their rank tables to the kernels as
+// kernel arguments; larger worlds go through the HBM tables (drank / crank),
+// written by bind kernels that take up to kBindBatch rows as arguments each.
+constexpr uint32_t kInlineRanks = 8;
 constexpr uint32_t kBindBatch = 16;
+// Steps with at most this many (token, pick) pairs dispatch in one fused launch.
+constexpr uint32_t kFusedMaxPairs = 16384;
+
 struct BindDispatchBatch {
   uint32_t first, count;
   uint64_t pad_;
@@ -90,12 +96,16 @@ struct BindCombineBatch {
   CombineRank rows[kBindBatch];
 };
 
-// Launchers implemented in a2a_kernels.hip; return a hipError_t as int.
+// Launchers implemented in a2a_kernels.hip; they return a hipError_t as int.
+// `inline_rows` (world_size rows, host memory) selects the inline-table kernels;
+// NULL selects the HBM tables, which must have been bound.
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream);
 int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stream);
-int launch_route(const WorldDev &w, void *stream);
-int launch_dispatch_scatter(const WorldDev &w, void *stream);
-int launch_combine_gather(const WorldDev &w, int in_dtype, int out_dtype, void *stream);
+int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *stream);
+int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
+                   void *stream);
+// True when dispatch runs as the single fused launch for this geometry.
+bool dispatch_is_fused(const WorldDev &w);
 // LDS bytes the routing kernels need for a given geometry.
 uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks);
 

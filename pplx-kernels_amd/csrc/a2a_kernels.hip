@@ -12,12 +12,18 @@
 //                    prefix over chunks and earlier tiles -> slot_map, counts
 //   dispatch_scatter one wave per token (or per share of its K picks): the row
 //                    is read once into registers and stored K times, 16 B / lane
+//   dispatch_fused   small steps: routing and scatter in one launch; every
+//                    workgroup recounts the picks of the tokens before its own
 //   combine_gather   one workgroup per token: K rows gathered through the slot
 //                    map, fp32 accumulate in pick order, 16 B stores
 //
-// No atomics on global memory, no spin waits, no cooperative launch: phase
-// boundaries are kernel boundaries on one stream, so a step captures into a
-// hipGraph as is.  Wavefronts are 64 wide throughout.
+// No atomics on global memory (fault flags aside), no spin waits, no
+// cooperative launch: phase boundaries are kernel boundaries on one stream, so a
+// step captures into a hipGraph as is.  Wavefronts are 64 wide throughout.
+//
+// Rank tables reach the kernels either inline, as kernel arguments (worlds of
+// up to kInlineRanks ranks: nothing to bind, nothing to go stale), or through
+// the HBM tables written by bind_rows.
 #include <hip/hip_runtime.h>
 
 #include "a2a_device.h"
@@ -31,14 +37,37 @@ typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+struct InlineDispatch {
+  DispatchRank rows[kInlineRanks];
+  __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
+};
+struct HbmDispatch {
+  const DispatchRank *rows;
+  __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
+};
+struct InlineCombine {
+  CombineRank rows[kInlineRanks];
+  __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
+};
+struct HbmCombine {
+  const CombineRank *rows;
+  __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
+};
+
 __device__ __forceinline__ uint32_t lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
 
+__device__ __forceinline__ uint64_t read_lane64(uint64_t v, uint32_t src_lane) {
+  return ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), (int)src_lane) << 32) |
+         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, (int)src_lane);
+}
+
 // Tokens present in DP group g this step: the reference's numSendTokens
 // (csrc/all_to_all/intranode_dispatch.cu:64), clamped to the rows that exist.
-__device__ __forceinline__ uint32_t dispatch_group_tokens(const WorldDev &w, uint32_t g) {
-  const DispatchRank &r = w.drank[g * w.dp];
+template <class DT>
+__device__ __forceinline__ uint32_t dispatch_group_tokens(const WorldDev &w, const DT &tab, uint32_t g) {
+  const DispatchRank &r = tab.at(g * w.dp);
   uint32_t n = r.bound_m ? *r.bound_m : r.m;
   n = n < r.m ? n : r.m;
   return n < w.M ? n : w.M;
@@ -69,7 +98,8 @@ __global__ __launch_bounds__(256) void bind_rows(Row *table, Batch b) {
 // the order in which the reference test appends to expert_token_from.  A tile
 // is tile_chunks consecutive chunks of 64 virtual tokens.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void route_count(WorldDev w) {
+template <class DT>
+__global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab) {
   extern __shared__ uint32_t lds_hist[];
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_hist[e] = 0;
   __syncthreads();
@@ -77,8 +107,8 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w) {
   const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  if (g < w.G && t < dispatch_group_tokens(w, g)) {
-    const uint32_t *idx = w.drank[g * w.dp + t % w.dp].indices + (size_t)t * w.K;
+  if (g < w.G && t < dispatch_group_tokens(w, tab, g)) {
+    const uint32_t *idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
       if (e < w.E) atomicAdd(&lds_hist[e], 1u);
@@ -89,7 +119,8 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w) {
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) out[e] = lds_hist[e];
 }
 
-__global__ __launch_bounds__(1024) void route_slots(WorldDev w) {
+template <class DT>
+__global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab) {
   // LDS: mask[chunks][E] (one bit per token of the chunk routed to e),
   //      then base[chunks][E] (rows of e taken before the chunk starts).
   extern __shared__ unsigned long long lds_mask[];
@@ -104,11 +135,11 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w) {
   const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  const bool live = g < w.G && t < dispatch_group_tokens(w, g);
+  const bool live = g < w.G && t < dispatch_group_tokens(w, tab, g);
   const uint32_t *idx = nullptr;
   bool bad_expert = false;
   if (live) {
-    idx = w.drank[g * w.dp + t % w.dp].indices + (size_t)t * w.K;
+    idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
       if (e < w.E) {
@@ -131,7 +162,7 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w) {
     if (blockIdx.x == gridDim.x - 1) {
       // out_expert_num_tokens of the owning rank
       // (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).
-      const DispatchRank &owner = w.drank[e / w.L];
+      const DispatchRank &owner = tab.at(e / w.L);
       owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
     }
   }
@@ -153,38 +184,34 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w) {
 }
 
 // ---------------------------------------------------------------------------
-// Dispatch scatter.  A wave owns one token and picks [k0, k1) of it.  NV is the
-// number of 16-byte vectors each lane keeps in registers (row <= NV * 1 KiB).
+// Row fan-out shared by dispatch_scatter and dispatch_fused.  The calling wave
+// owns token (g, t); lane k passes the slot of pick k in `slot`.  The row is
+// read once into NV 16-byte registers per lane and stored for picks [k0, k1).
+// EXACT: the row is exactly NV * 64 vectors, so nothing is predicated.
 // ---------------------------------------------------------------------------
-template <int NV>
-__global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, uint32_t ksplit, uint32_t kper) {
-  const uint32_t lane = lane_id();
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
-                                                       threadIdx.x / kWave);
-  const uint32_t v = wave / ksplit;
-  const uint32_t part = wave - v * ksplit;
-  const uint32_t g = v / w.M;
-  const uint32_t t = v - g * w.M;
-  if (g >= w.G) return;
-  if (t >= dispatch_group_tokens(w, g)) return;
-
+template <int NV, bool EXACT, class DT>
+__device__ __forceinline__ void fan_out_row(const WorldDev &w, const DT &tab, uint32_t g, uint32_t t,
+                                            uint32_t lane, uint32_t slot, uint32_t k0, uint32_t k1,
+                                            bool report) {
   // The sender of token t inside its DP group (csrc/all_to_all/intranode_dispatch.cu:97).
-  const DispatchRank &src = w.drank[g * w.dp + t % w.dp];
+  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
   const uint32_t nvec = w.Hb / 16;
   const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
 
   u32x4 x[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const uint32_t j = lane + i * kWave;
-    if (j < nvec) x[i] = row[j];
+    uint32_t j = lane + i * kWave;
+    if (!EXACT) j = j < nvec ? j : nvec - 1;  // clamp: loads stay unconditional
+    x[i] = row[j];
   }
   const uint32_t S = w.S;
   const float *srow = nullptr;
   float sc = 0.f;
   if (S) {
     srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
-    if (lane < S) sc = srow[(int64_t)lane * src.dp_xs_stride_elem];
+    const uint32_t j = lane < S ? lane : S - 1;
+    sc = srow[(int64_t)j * src.dp_xs_stride_elem];
   }
 
   // Lane k resolves the destination of pick k.
@@ -192,9 +219,8 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, uint32_t ksp
   int64_t dst_scale_step = 0;
   if (lane < w.K) {
     const uint32_t e = src.indices[(size_t)t * w.K + lane];
-    const uint32_t slot = w.slot_map[(size_t)v * w.K + lane];
     if (e < w.E && slot != kInvalidSlot) {
-      const DispatchRank &dst = w.drank[e / w.L];
+      const DispatchRank &dst = tab.at(e / w.L);
       const uint32_t el = e % w.L;
       if (slot < dst.x_rows) {
         dst_row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
@@ -204,32 +230,24 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, uint32_t ksp
                                                  (int64_t)slot * dst.xs_stride_row);
           dst_scale_step = dst.xs_stride_elem;
         }
-      } else if (part == 0) {
+      } else if (report) {
         atomicOr(w.faults, kFaultRowDropped);
       }
     }
   }
 
-  const uint32_t k0 = part * kper;
-  const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
   for (uint32_t k = k0; k < k1; ++k) {
-    const uint64_t p = ((uint64_t)__builtin_amdgcn_readlane((uint32_t)(dst_row >> 32), k) << 32) |
-                       (uint32_t)__builtin_amdgcn_readlane((uint32_t)dst_row, k);
+    const uint64_t p = read_lane64(dst_row, k);
     if (p == 0) continue;
     u32x4 *out = reinterpret_cast<u32x4 *>(p);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const uint32_t j = lane + i * kWave;
-      if (j < nvec) __builtin_nontemporal_store(x[i], out + j);
+      if (EXACT || j < nvec) __builtin_nontemporal_store(x[i], out + j);
     }
     if (S) {
-      const uint64_t q = ((uint64_t)__builtin_amdgcn_readlane((uint32_t)(dst_scale >> 32), k) << 32) |
-                         (uint32_t)__builtin_amdgcn_readlane((uint32_t)dst_scale, k);
-      const uint64_t step64 =
-          ((uint64_t)__builtin_amdgcn_readlane((uint32_t)((uint64_t)dst_scale_step >> 32), k) << 32) |
-          (uint32_t)__builtin_amdgcn_readlane((uint32_t)dst_scale_step, k);
-      float *sout = reinterpret_cast<float *>(q);
-      const int64_t step = (int64_t)step64;
+      float *sout = reinterpret_cast<float *>(read_lane64(dst_scale, k));
+      const int64_t step = (int64_t)read_lane64((uint64_t)dst_scale_step, k);
       if (lane < S) sout[(int64_t)lane * step] = sc;
       for (uint32_t j = lane + kWave; j < S; j += kWave) {
         sout[(int64_t)j * step] = srow[(int64_t)j * src.dp_xs_stride_elem];
@@ -238,8 +256,105 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, uint32_t ksp
   }
 }
 
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+  const uint32_t lane = lane_id();
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
+                                                       threadIdx.x / kWave);
+  const uint32_t v = wave / ksplit;
+  const uint32_t part = wave - v * ksplit;
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (g >= w.G) return;
+  if (t >= dispatch_group_tokens(w, tab, g)) return;
+  const uint32_t slot = lane < w.K ? w.slot_map[(size_t)v * w.K + lane] : kInvalidSlot;
+  const uint32_t k0 = part * kper;
+  const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
+  fan_out_row<NV, EXACT>(w, tab, g, t, lane, slot, k0, k1, part == 0);
+}
+
+// Small steps: one launch does routing and scatter.  A workgroup owns
+// tokens_per_block consecutive virtual tokens.  It first counts, per expert, the
+// picks of all tokens before its own (every workgroup repeats this over the
+// indices, which are a few KiB in L2), then assigns its own tokens' slots in
+// order, then fans the rows out.  The last workgroup has counted everything
+// and writes out_expert_num_tokens.
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+  extern __shared__ uint32_t lds_u32[];
+  uint32_t *hist = lds_u32;             // [E]
+  uint32_t *ntok = hist + w.E;          // [G]
+  uint32_t *own_slot = ntok + w.G;      // [tokens_per_block][K]
+  const uint32_t waves = blockDim.x / kWave;
+  const uint32_t tokens_per_block = waves / ksplit;
+
+  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) hist[e] = 0;
+  for (uint32_t g = threadIdx.x; g < w.G; g += blockDim.x) ntok[g] = dispatch_group_tokens(w, tab, g);
+  __syncthreads();
+
+  const uint32_t v0 = blockIdx.x * tokens_per_block;
+  bool bad_expert = false;
+  for (uint32_t v = threadIdx.x; v < v0; v += blockDim.x) {
+    const uint32_t g = v / w.M;
+    const uint32_t t = v - g * w.M;
+    if (t < ntok[g]) {
+      const uint32_t *idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
+      for (uint32_t k = 0; k < w.K; ++k) {
+        const uint32_t e = idx[k];
+        if (e < w.E) atomicAdd(&hist[e], 1u);
+      }
+    }
+  }
+  __syncthreads();
+
+  const uint32_t total = w.G * w.M;
+  for (uint32_t j = 0; j < tokens_per_block; ++j) {
+    const uint32_t v = v0 + j;
+    if (v < total && threadIdx.x < w.K) {
+      const uint32_t g = v / w.M;
+      const uint32_t t = v - g * w.M;
+      uint32_t slot = kInvalidSlot;
+      if (t < ntok[g]) {
+        const uint32_t e = tab.at(g * w.dp + t % w.dp).indices[(size_t)t * w.K + threadIdx.x];
+        if (e < w.E) {
+          slot = hist[e];  // experts of one token are distinct: no two threads share e
+          hist[e] = slot + 1;
+        } else {
+          bad_expert = true;
+        }
+        w.slot_map[(size_t)v * w.K + threadIdx.x] = slot;
+      }
+      own_slot[j * w.K + threadIdx.x] = slot;
+    }
+    __syncthreads();
+  }
+  if (bad_expert) atomicOr(w.faults, kFaultBadExpert);
+
+  if (blockIdx.x == gridDim.x - 1) {
+    for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
+      const DispatchRank &owner = tab.at(e / w.L);
+      owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
+    }
+  }
+
+  const uint32_t lane = lane_id();
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t j = wave / ksplit;
+  const uint32_t part = wave - j * ksplit;
+  const uint32_t v = v0 + j;
+  if (j >= tokens_per_block || v >= total) return;
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (t >= ntok[g]) return;
+  const uint32_t slot = lane < w.K ? own_slot[j * w.K + lane] : kInvalidSlot;
+  const uint32_t k0 = part * kper;
+  const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
+  fan_out_row<NV, EXACT>(w, tab, g, t, lane, slot, k0, k1, part == 0);
+}
+
 // Rows longer than the register variants cover: stream each vector K times.
-__global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w) {
+template <class DT>
+__global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab) {
   __shared__ uint64_t s_row[kWave];
   __shared__ uint64_t s_scale[kWave];
   __shared__ int64_t s_step[kWave];
@@ -247,15 +362,15 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w) {
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
-  if (t >= dispatch_group_tokens(w, g)) return;
-  const DispatchRank &src = w.drank[g * w.dp + t % w.dp];
+  if (t >= dispatch_group_tokens(w, tab, g)) return;
+  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
   if (threadIdx.x < w.K) {
     uint64_t dst_row = 0, dst_scale = 0;
     int64_t step = 0;
     const uint32_t e = src.indices[(size_t)t * w.K + threadIdx.x];
     const uint32_t slot = w.slot_map[(size_t)v * w.K + threadIdx.x];
     if (e < w.E && slot != kInvalidSlot) {
-      const DispatchRank &dst = w.drank[e / w.L];
+      const DispatchRank &dst = tab.at(e / w.L);
       const uint32_t el = e % w.L;
       if (slot < dst.x_rows) {
         dst_row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
@@ -298,18 +413,25 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w) {
 // with k ascending and fp32 accumulation
 // (csrc/all_to_all/intranode_combine.cu:141-168).
 // ---------------------------------------------------------------------------
-template <typename T> struct Load8;
-template <> struct Load8<float> {
-  static __device__ __forceinline__ f32x8 at(const void *row, uint32_t vec) {
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+  struct Raw {
+    f32x4 a, b;
+  };
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
     const f32x4 *p = reinterpret_cast<const f32x4 *>(row) + 2 * (size_t)vec;
-    const f32x4 a = __builtin_nontemporal_load(p);
-    const f32x4 b = __builtin_nontemporal_load(p + 1);
-    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+    return Raw{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1)};
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &r) {
+    return __builtin_shufflevector(r.a, r.b, 0, 1, 2, 3, 4, 5, 6, 7);
   }
 };
-template <> struct Load8<__bf16> {
-  static __device__ __forceinline__ f32x8 at(const void *row, uint32_t vec) {
-    const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + vec);
+template <> struct Row8<__bf16> {
+  typedef u32x4 Raw;
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + vec);
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
     f32x8 out;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -319,9 +441,12 @@ template <> struct Load8<__bf16> {
     return out;
   }
 };
-template <> struct Load8<_Float16> {
-  static __device__ __forceinline__ f32x8 at(const void *row, uint32_t vec) {
-    const f16x8 raw = __builtin_nontemporal_load(reinterpret_cast<const f16x8 *>(row) + vec);
+template <> struct Row8<_Float16> {
+  typedef f16x8 Raw;
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
+    return __builtin_nontemporal_load(reinterpret_cast<const f16x8 *>(row) + vec);
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
     return __builtin_convertvector(raw, f32x8);
   }
 };
@@ -338,50 +463,186 @@ template <> struct Store8<_Float16> {
   }
 };
 
-template <typename T, typename U>
-__global__ __launch_bounds__(256) void combine_gather(WorldDev w) {
-  __shared__ uint64_t s_row[kWave];
-  __shared__ float s_weight[kWave];
+// N picks starting at k: all N loads are issued before the first is used.
+template <typename T, int N>
+__device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, float weight_of_lane,
+                                             uint32_t k, uint32_t vec) {
+  typename Row8<T>::Raw raw[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) raw[i] = Row8<T>::load(read_lane64(row_of_lane, k + i), vec);
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float wk = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight_of_lane), (int)(k + i)));
+    acc += wk * Row8<T>::widen(raw[i]);
+  }
+}
 
+template <typename T, typename U, class CT>
+__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab) {
   const uint32_t r = blockIdx.x / w.M;
   const uint32_t t = blockIdx.x - r * w.M;
-  const CombineRank &c = w.crank[r];
+  const CombineRank &c = tab.at(r);
   if (t >= combine_rank_tokens(w, c)) return;
 
-  if (threadIdx.x < w.K) {
-    const uint32_t k = threadIdx.x;
-    const uint32_t e = c.indices[(size_t)t * w.K + k];
-    const uint32_t slot = w.slot_map[((size_t)(r / w.dp) * w.M + t) * w.K + k];
-    uint64_t p = 0;
+  // Every wave resolves the K picks itself (lane k <-> pick k): no LDS, no barrier.
+  const uint32_t lane = lane_id();
+  uint64_t row = 0;
+  float weight = 0.f;
+  if (lane < w.K) {
+    const uint32_t e = c.indices[(size_t)t * w.K + lane];
+    const uint32_t slot = w.slot_map[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
+    weight = c.weights[(int64_t)t * c.w_stride_row + lane];
     if (e < w.E && slot != kInvalidSlot) {
-      const CombineRank &owner = w.crank[e / w.L];
+      const CombineRank &owner = tab.at(e / w.L);
       if (slot < owner.y_rows) {
-        p = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
-                                       (int64_t)(e % w.L) * owner.y_stride_expert +
-                                       (int64_t)slot * owner.y_stride_row);
-      } else {
+        row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
+                                         (int64_t)(e % w.L) * owner.y_stride_expert +
+                                         (int64_t)slot * owner.y_stride_row);
+      } else if (threadIdx.x == lane) {
         atomicOr(w.faults, kFaultBadSlot);
       }
     }
-    s_row[k] = p;
-    s_weight[k] = c.weights[(int64_t)t * c.w_stride_row + k];
   }
-  __syncthreads();
+  const bool all_rows = __builtin_amdgcn_ballot_w64(lane < w.K && row == 0) == 0;
 
   U *out = reinterpret_cast<U *>(c.out_tokens) + (int64_t)t * c.out_stride_row;
   const uint32_t nvec = w.H / 8;
-  for (uint32_t vec = threadIdx.x; vec < nvec; vec += blockDim.x) {
-    f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-    for (uint32_t k = 0; k < w.K; ++k) {
-      const uint64_t p = s_row[k];
-      if (p == 0) continue;
-      const float wk = s_weight[k];
-      const f32x8 y = Load8<T>::at(reinterpret_cast<const void *>(p), vec);
-      acc += wk * y;
+  const uint32_t K = w.K;
+  if (all_rows) {
+    for (uint32_t vec = threadIdx.x; vec < nvec; vec += blockDim.x) {
+      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      uint32_t k = 0;
+      for (; k + 8 <= K; k += 8) gather_group<T, 8>(acc, row, weight, k, vec);
+      if (K & 4) { gather_group<T, 4>(acc, row, weight, k, vec); k += 4; }
+      if (K & 2) { gather_group<T, 2>(acc, row, weight, k, vec); k += 2; }
+      if (K & 1) { gather_group<T, 1>(acc, row, weight, k, vec); }
+      Store8<U>::at(out, vec, acc);
     }
-    Store8<U>::at(out, vec, acc);
+  } else {
+    // A pick without a row (bad expert id or slot) contributes nothing.
+    for (uint32_t vec = threadIdx.x; vec < nvec; vec += blockDim.x) {
+      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (uint32_t k = 0; k < K; ++k) {
+        if (read_lane64(row, k) != 0) gather_group<T, 1>(acc, row, weight, k, vec);
+      }
+      Store8<U>::at(out, vec, acc);
+    }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Launch helpers
+// ---------------------------------------------------------------------------
+InlineDispatch make_inline(const WorldDev &w, const DispatchRank *rows) {
+  InlineDispatch t{};
+  for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
+  return t;
+}
+
+InlineCombine make_inline(const WorldDev &w, const CombineRank *rows) {
+  InlineCombine t{};
+  for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
+  return t;
+}
+
+template <class DT>
+int launch_route_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+  const uint32_t block = w.tile_chunks * kWave;
+  if (w.num_tiles > 1) {
+    hipLaunchKernelGGL(route_count<DT>, dim3(w.num_tiles), dim3(block), w.E * sizeof(uint32_t), s, w, tab);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return (int)err;
+  }
+  hipLaunchKernelGGL(route_slots<DT>, dim3(w.num_tiles), dim3(block), route_lds_bytes(w.E, w.tile_chunks),
+                     s, w, tab);
+  return (int)hipGetLastError();
+}
+
+// Picks the register variant for the row size and launches KERNEL<NV, EXACT, DT>.
+#define PPLX_LAUNCH_ROW_VARIANT(KERNEL, NV, EXACT)                                               \
+  hipLaunchKernelGGL((KERNEL<NV, EXACT, DT>), grid, block, lds, s, w, tab, ksplit, kper)
+
+#define PPLX_DISPATCH_ROW_VARIANTS(KERNEL)                                                       \
+  do {                                                                                           \
+    const uint32_t nvec = w.Hb / 16;                                                             \
+    const uint32_t per_lane = (nvec + kWave - 1) / kWave;                                        \
+    const bool exact = nvec % kWave == 0;                                                        \
+    if (exact && per_lane == 1) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 1, true);                        \
+    else if (exact && per_lane == 2) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 2, true);                   \
+    else if (exact && per_lane == 3) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 3, true);                   \
+    else if (exact && per_lane == 4) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 4, true);                   \
+    else if (exact && per_lane == 5) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 5, true);                   \
+    else if (exact && per_lane == 6) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 6, true);                   \
+    else if (exact && per_lane == 7) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 7, true);                   \
+    else if (exact && per_lane == 8) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 8, true);                   \
+    else if (per_lane <= 1) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 1, false);                           \
+    else if (per_lane <= 2) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 2, false);                           \
+    else if (per_lane <= 4) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 4, false);                           \
+    else if (per_lane <= 8) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 8, false);                           \
+    else if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                         \
+    else PPLX_LAUNCH_ROW_VARIANT(KERNEL, 32, false);                                             \
+  } while (0)
+
+// Number of waves a row's K copies are spread over: few tokens -> more waves,
+// so that the launch still covers the 256 CUs (the row re-reads hit L2).
+uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
+  const uint64_t tokens = (uint64_t)w.G * w.M;
+  uint32_t ksplit = 1;
+  while (ksplit < max_split && ksplit < w.K && tokens * ksplit < 4096) ksplit *= 2;
+  return ksplit;
+}
+
+template <class DT>
+int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+  const uint32_t tokens = w.G * w.M;
+  if ((w.Hb / 16 + kWave - 1) / kWave > 32) {
+    hipLaunchKernelGGL(dispatch_scatter_long<DT>, dim3(tokens), dim3(256), 0, s, w, tab);
+    return (int)hipGetLastError();
+  }
+  const uint32_t ksplit = pick_ksplit(w, kWave);
+  const uint32_t kper = (w.K + ksplit - 1) / ksplit;
+  const uint64_t waves = (uint64_t)tokens * ksplit;
+  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
+  const uint32_t lds = 0;
+  PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
+  return (int)hipGetLastError();
+}
+
+template <class DT>
+int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+  const uint32_t tokens = w.G * w.M;
+  const uint32_t ksplit = pick_ksplit(w, 4);  // 4 waves per workgroup
+  const uint32_t kper = (w.K + ksplit - 1) / ksplit;
+  const uint32_t tokens_per_block = 4 / ksplit;
+  const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(256);
+  const uint32_t lds = (w.E + w.G + tokens_per_block * w.K) * sizeof(uint32_t);
+  PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
+  return (int)hipGetLastError();
+}
+
+template <class DT>
+int launch_dispatch_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+  if (dispatch_is_fused(w)) return launch_fused_t(w, tab, s);
+  int err = launch_route_t(w, tab, s);
+  if (err) return err;
+  return launch_scatter_t(w, tab, s);
+}
+
+template <class CT>
+int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s) {
+  const dim3 grid(w.R * w.M), block(256);
+  // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
+  switch (in_dtype * 4 + out_dtype) {
+    case 0 * 4 + 1: hipLaunchKernelGGL((combine_gather<float, __bf16, CT>), grid, block, 0, s, w, tab); break;
+    case 0 * 4 + 2: hipLaunchKernelGGL((combine_gather<float, _Float16, CT>), grid, block, 0, s, w, tab); break;
+    case 1 * 4 + 1: hipLaunchKernelGGL((combine_gather<__bf16, __bf16, CT>), grid, block, 0, s, w, tab); break;
+    case 1 * 4 + 2: hipLaunchKernelGGL((combine_gather<__bf16, _Float16, CT>), grid, block, 0, s, w, tab); break;
+    case 2 * 4 + 1: hipLaunchKernelGGL((combine_gather<_Float16, __bf16, CT>), grid, block, 0, s, w, tab); break;
+    case 2 * 4 + 2: hipLaunchKernelGGL((combine_gather<_Float16, _Float16, CT>), grid, block, 0, s, w, tab); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  return (int)hipGetLastError();
 }
 
 }  // namespace
@@ -391,6 +652,14 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w) {
 // ---------------------------------------------------------------------------
 uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
   return tile_chunks * num_experts * (uint32_t)(sizeof(unsigned long long) + sizeof(uint32_t));
+}
+
+bool dispatch_is_fused(const WorldDev &w) {
+  // Every workgroup recounts all earlier picks, so the one-launch form only pays
+  // while the whole step's routing is a few tens of KiB.
+  const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
+  const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
+  return pairs <= kFusedMaxPairs && per_lane <= 32 && (w.E + w.G + 4 * w.K) * 4 <= 48 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {
@@ -405,65 +674,16 @@ int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stre
   return (int)hipGetLastError();
 }
 
-int launch_route(const WorldDev &w, void *stream) {
-  const uint32_t block = w.tile_chunks * kWave;
-  if (w.num_tiles > 1) {
-    hipLaunchKernelGGL(route_count, dim3(w.num_tiles), dim3(block), w.E * sizeof(uint32_t),
-                       (hipStream_t)stream, w);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) return (int)err;
-  }
-  hipLaunchKernelGGL(route_slots, dim3(w.num_tiles), dim3(block),
-                     route_lds_bytes(w.E, w.tile_chunks), (hipStream_t)stream, w);
-  return (int)hipGetLastError();
+int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *stream) {
+  if (inline_rows) return launch_dispatch_t(w, make_inline(w, inline_rows), (hipStream_t)stream);
+  return launch_dispatch_t(w, HbmDispatch{w.drank}, (hipStream_t)stream);
 }
 
-int launch_dispatch_scatter(const WorldDev &w, void *stream) {
-  const uint32_t tokens = w.G * w.M;
-  const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
-  if (per_lane > 32) {
-    hipLaunchKernelGGL(dispatch_scatter_long, dim3(tokens), dim3(256), 0, (hipStream_t)stream, w);
-    return (int)hipGetLastError();
-  }
-  // Few tokens: spread the K copies of a row over several waves so the launch
-  // still covers the 256 CUs; the row re-reads hit L2.
-  uint32_t ksplit = 1;
-  while (ksplit < w.K && (uint64_t)tokens * ksplit < 16384) ksplit *= 2;
-  if (ksplit > w.K) ksplit = w.K;
-  const uint32_t kper = (w.K + ksplit - 1) / ksplit;
-  const uint64_t waves = (uint64_t)tokens * ksplit;
-  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
-  hipStream_t s = (hipStream_t)stream;
-  if (per_lane <= 1) {
-    hipLaunchKernelGGL(dispatch_scatter<1>, grid, block, 0, s, w, ksplit, kper);
-  } else if (per_lane <= 2) {
-    hipLaunchKernelGGL(dispatch_scatter<2>, grid, block, 0, s, w, ksplit, kper);
-  } else if (per_lane <= 4) {
-    hipLaunchKernelGGL(dispatch_scatter<4>, grid, block, 0, s, w, ksplit, kper);
-  } else if (per_lane <= 8) {
-    hipLaunchKernelGGL(dispatch_scatter<8>, grid, block, 0, s, w, ksplit, kper);
-  } else if (per_lane <= 16) {
-    hipLaunchKernelGGL(dispatch_scatter<16>, grid, block, 0, s, w, ksplit, kper);
-  } else {
-    hipLaunchKernelGGL(dispatch_scatter<32>, grid, block, 0, s, w, ksplit, kper);
-  }
-  return (int)hipGetLastError();
-}
-
-int launch_combine_gather(const WorldDev &w, int in_dtype, int out_dtype, void *stream) {
-  const dim3 grid(w.R * w.M), block(256);
-  hipStream_t s = (hipStream_t)stream;
-  // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
-  switch (in_dtype * 4 + out_dtype) {
-    case 0 * 4 + 1: hipLaunchKernelGGL((combine_gather<float, __bf16>), grid, block, 0, s, w); break;
-    case 0 * 4 + 2: hipLaunchKernelGGL((combine_gather<float, _Float16>), grid, block, 0, s, w); break;
-    case 1 * 4 + 1: hipLaunchKernelGGL((combine_gather<__bf16, __bf16>), grid, block, 0, s, w); break;
-    case 1 * 4 + 2: hipLaunchKernelGGL((combine_gather<__bf16, _Float16>), grid, block, 0, s, w); break;
-    case 2 * 4 + 1: hipLaunchKernelGGL((combine_gather<_Float16, __bf16>), grid, block, 0, s, w); break;
-    case 2 * 4 + 2: hipLaunchKernelGGL((combine_gather<_Float16, _Float16>), grid, block, 0, s, w); break;
-    default: return (int)hipErrorInvalidValue;
-  }
-  return (int)hipGetLastError();
+int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
+                   void *stream) {
+  if (inline_rows)
+    return launch_combine_t(w, make_inline(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream);
+  return launch_combine_t(w, HbmCombine{w.crank}, in_dtype, out_dtype, (hipStream_t)stream);
 }
 
 }  // namespace pplx_amd

@@ -183,6 +183,17 @@ class _World:
         self.cfg = cfg_tuple
         self.ptr = ptr
         self.handles: set[int] = set()
+        self.world_size = cfg_tuple[3]
+        # A step's kernels are enqueued by the last rank to call, so the tensors of the
+        # ranks that called earlier are kept alive until then: a temporary such as
+        # ``x.to(device)`` must not go back to the caching allocator before it is read.
+        self.pending: dict[str, list] = {"dispatch": [], "combine": []}
+
+    def hold(self, kind: str, tensors: tuple) -> None:
+        held = self.pending[kind]
+        held.append(tensors)
+        if len(held) >= self.world_size:
+            held.clear()
 
 
 _worlds: dict[str, _World] = {}
@@ -478,6 +489,10 @@ def _dispatch(
     mode = split_mode(do_send, do_recv)
     with torch.cuda.device(indices.device):
         check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
+    _handle_world[fptr].hold(
+        "dispatch",
+        (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
+    )
 
 
 def _combine(
@@ -495,6 +510,7 @@ def _combine(
     mode = split_mode(do_send, do_recv)
     with torch.cuda.device(indices.device):
         check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
+    _handle_world[fptr].hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
 
 
 def _fake_dispatch(*args, **kwargs) -> None:

@@ -339,3 +339,55 @@ def make_world(spec: WorkloadSpec, group_name: str = "loopback"):
         spec.hidden_dim_scale_bytes,
         group_name,
     )
+
+
+# ---------------------------------------------------------------------------
+# Comparison of a device step with the CPU oracle
+# ---------------------------------------------------------------------------
+def check_dispatch_against_oracle(step: DeviceStep, expected=None):
+    """Bit-exact comparison of counts, rows and scale bits (rows beyond an expert's count
+    are unconstrained).  Returns the oracle's DispatchResult."""
+    from oracle import a2a_oracle as orc
+
+    s = step.spec
+    E, K, M = s.num_experts, s.experts_per_token, s.max_num_tokens
+    if expected is None:
+        expected = orc.c_dispatch(to_oracle_groups(step.groups), M, E, K, step.cap)
+    torch.cuda.synchronize()
+    counts = step.expert_num_tokens_all.cpu().numpy().reshape(E)
+    np.testing.assert_array_equal(counts, expected.counts)
+    live = np.arange(step.cap)[None, :] < expected.counts[:, None]
+    got_x = step.expert_x_all.view(torch.uint8).reshape(E, step.cap, -1).cpu().numpy()
+    np.testing.assert_array_equal(got_x[live], expected.expert_x[live])
+    if s.scale_dim:
+        got_s = step.expert_x_scale_all.reshape(E, step.cap, -1).cpu().numpy()
+        np.testing.assert_array_equal(got_s[live].view(np.uint32), expected.expert_x_scale[live].view(np.uint32))
+    return expected
+
+
+COMBINE_RTOL = 1e-2  # bf16 tolerance of the fp32-accumulated reference
+COMBINE_ATOL = 1e-2
+
+
+def check_combine_against_oracle(step: DeviceStep, slot_map: np.ndarray, use_numpy: bool = False):
+    """out_tokens[:n] within rtol 1e-2 / atol 1e-2 of the fp32-accumulated oracle; rows >= n
+    still hold the NaN they were filled with."""
+    from oracle import a2a_oracle as orc
+
+    s = step.spec
+    E, K, M, H = s.num_experts, s.experts_per_token, s.max_num_tokens, s.hidden_dim
+    torch.cuda.synchronize()
+    y = torch_bits(step.expert_y_all.reshape(E, step.cap, H))
+    in_dt, out_dt = ORACLE_DTYPE[s.expert_y_dtype], ORACLE_DTYPE[s.out_dtype]
+    fn = orc.np_combine if use_numpy else orc.c_combine
+    want = fn(to_oracle_groups(step.groups), M, E, K, H, y, in_dt, out_dt, slot_map)
+    for r in range(s.world_size):
+        g = step.groups[r // s.dp_size]
+        got = step.out_tokens[r].cpu()
+        w = orc.to_float32(want[r // s.dp_size], out_dt)
+        np.testing.assert_allclose(
+            got[: g.n].float().numpy(), w, rtol=COMBINE_RTOL, atol=COMBINE_ATOL,
+            err_msg=f"combine mismatch on rank {r}",
+        )  # fmt: skip
+        assert torch.isnan(got[g.n :]).all(), f"rank {r}: rows >= bound_m were written"
+    return want

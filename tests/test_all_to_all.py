@@ -1,0 +1,551 @@
+"""GPU parity tests of the HIP dispatch / combine path against the CPU oracle.
+
+Everything here goes through the C ABI (``libpplx_kernels.so``) via the ``pplx_kernels``
+Python surface.  Structure follows the reference's ``tests/test_all_to_all.py``: the same
+call sequence and keyword arguments (``:180-190,264-270``), the same property checks
+(``:196-246,277-286``), plus bit-exact comparison with the oracle, which the reference's
+nondeterministic slot assignment could not offer.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests.all_to_all_utils import (
+    COMBINE_ATOL,
+    COMBINE_RTOL,
+    FP8,
+    DeviceStep,
+    GroupInputs,
+    MoEConfig,
+    RankTestData,
+    WorkloadSpec,
+    baseline_configs,
+    check_combine_against_oracle,
+    check_dispatch_against_oracle,
+    expert_counts,
+    generate,
+    make_world,
+    small_moe,
+)
+
+pytestmark = pytest.mark.gpu
+
+
+def spec_from_moe(cfg: MoEConfig, world_size: int, dp_size: int, name: str = "ref") -> WorkloadSpec:
+    return WorkloadSpec(
+        name, 0, world_size, cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim,
+        cfg.max_num_tokens, cfg.in_dtype, out_dtype=cfg.out_dtype, expert_y_dtype=cfg.out_dtype,
+        dp_size=dp_size,
+    )  # fmt: skip
+
+
+def run_and_check(spec, groups, *, api="world", cap=None, with_bound_m=True, y_seed=0, use_numpy=False):
+    """dispatch -> check -> random expert_y -> combine -> check; returns the DeviceStep."""
+    from pplx_kernels import AllToAll
+
+    step = DeviceStep(spec, groups, cap=cap, with_bound_m=with_bound_m)
+    name = f"t-{spec.name}-{api}"
+    if api == "world":
+        world = make_world(spec, group_name=name)
+        step.dispatch_world(world)
+    else:
+        ranks = [
+            AllToAll.intranode(
+                max_num_tokens=spec.max_num_tokens,
+                num_experts=spec.num_experts,
+                experts_per_token=spec.experts_per_token,
+                rank=r,
+                world_size=spec.world_size,
+                dp_size=spec.dp_size,
+                hidden_dim=spec.hidden_dim,
+                hidden_dim_bytes=spec.hidden_dim_bytes,
+                hidden_dim_scale_bytes=spec.hidden_dim_scale_bytes,
+                group_name=name,
+            )
+            for r in range(spec.world_size)
+        ]
+        step.dispatch_per_rank(ranks)
+    expected = check_dispatch_against_oracle(step)
+    gen = torch.Generator(device="cuda").manual_seed(y_seed)
+    step.expert_y_all.copy_(
+        torch.randn(step.expert_y_all.shape, generator=gen, device="cuda", dtype=torch.float32)
+    )
+    if api == "world":
+        step.combine_world(world)
+        assert world.faults() == 0
+        world.destroy()
+    else:
+        step.combine_per_rank(ranks)
+        for a in ranks:
+            a.destroy()
+    check_combine_against_oracle(step, expected.slot_map, use_numpy=use_numpy)
+    return step
+
+
+# ---------------------------------------------------------------------------
+# The reference's own test, restated for the loopback (world 4, dp 2, small_moe)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("in_dtype", ["bfloat16", "float8_e4m3fn", "float16"])
+@pytest.mark.parametrize("out_dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("internode", [True, False])
+def test_all_to_all_reference_flow(in_dtype, out_dtype, internode):
+    """tests/test_all_to_all.py:48-286 with every rank in this process."""
+    from pplx_kernels import AllToAll
+
+    world_size, dp_size = 4, 2
+    moe = dataclasses.replace(small_moe, in_dtype=getattr(torch, in_dtype), out_dtype=getattr(torch, out_dtype))
+    num_dp = world_size // dp_size
+    device = torch.device("cuda:0")
+    scale_bytes = 0 if moe.in_dtype.itemsize != 1 else moe.scale_dim * 4
+    make = AllToAll.internode if internode else AllToAll.intranode
+    atas = [
+        make(
+            max_num_tokens=moe.max_num_tokens,
+            num_experts=moe.num_experts,
+            experts_per_token=moe.experts_per_token,
+            rank=rank,
+            world_size=world_size,
+            dp_size=dp_size,
+            hidden_dim=moe.hidden_dim,
+            hidden_dim_bytes=moe.hidden_dim * moe.in_dtype.itemsize,
+            hidden_dim_scale_bytes=scale_bytes,
+        )
+        for rank in range(world_size)
+    ]
+    rng = torch.Generator()
+    rng.manual_seed(123)
+    all_rank_data = [RankTestData(moe, rng, use_max_tokens=False) for _ in range(num_dp)]
+    expert_token_from = [[] for _ in range(moe.num_experts)]
+    for i_rank, rd in enumerate(all_rank_data):
+        for token_idx in range(rd.num_tokens):
+            for expert_idx in rd.indices[token_idx]:
+                expert_token_from[expert_idx].append((i_rank, token_idx))
+
+    num_local_experts = moe.num_experts // world_size
+    outs = []
+    for rank, ata in enumerate(atas):
+        rank_data = all_rank_data[rank // dp_size]
+        expert_num_tokens = torch.empty(num_local_experts, dtype=torch.int32, device=device)
+        expert_x = torch.empty(
+            (num_local_experts, moe.max_num_tokens * num_dp, moe.hidden_dim), dtype=moe.in_dtype, device=device
+        )
+        expert_x_scale = None
+        if moe.in_dtype.itemsize == 1:
+            expert_x_scale = torch.empty(
+                (num_local_experts, expert_x.size(1), moe.scale_dim), dtype=torch.float32, device=device
+            )
+        bound_m = torch.tensor([rank_data.num_tokens], dtype=torch.uint32, device=device)
+        ata.dispatch(
+            out_expert_num_tokens=expert_num_tokens,
+            out_expert_x=expert_x,
+            out_expert_x_scale=expert_x_scale,
+            dp_x=rank_data.x.to(device),
+            dp_x_scale=rank_data.x_scale.to(device) if rank_data.x_scale is not None else None,
+            indices=rank_data.indices.to(device).to(torch.uint32),
+            bound_m=bound_m,
+        )
+        outs.append((expert_num_tokens, expert_x, expert_x_scale, bound_m))
+    torch.cuda.synchronize()
+
+    for rank in range(world_size):
+        expert_num_tokens, expert_x, expert_x_scale, _ = outs[rank]
+        for i_local_expert in range(num_local_experts):
+            expert_idx = rank * num_local_experts + i_local_expert
+            cnt_tokens = int(expert_num_tokens[i_local_expert].item())
+            assert cnt_tokens == len(expert_token_from[expert_idx])
+            for i_token in range(cnt_tokens):
+                # stronger than the reference's set equality: the exact canonical position
+                src_dp_rank, src_token_idx = expert_token_from[expert_idx][i_token]
+                src = all_rank_data[src_dp_rank]
+                assert torch.equal(
+                    expert_x[i_local_expert, i_token].cpu().view(torch.uint8),
+                    src.x[src_token_idx].view(torch.uint8),
+                )
+                if expert_x_scale is not None:
+                    assert torch.equal(expert_x_scale[i_local_expert, i_token].cpu(), src.x_scale[src_token_idx])
+
+    val = 1.5
+    ys = []
+    for rank, ata in enumerate(atas):
+        rank_data = all_rank_data[rank // dp_size]
+        _, expert_x, _, bound_m = outs[rank]
+        expert_y = expert_x.to(moe.out_dtype) * val
+        y = torch.full((moe.max_num_tokens, moe.hidden_dim), torch.nan, dtype=moe.out_dtype, device=device)
+        ata.combine(
+            out_tokens=y,
+            indices=rank_data.indices.to(device).to(torch.uint32),
+            weights=rank_data.weights.to(device),
+            expert_y=expert_y,
+            bound_m=bound_m,
+        )
+        ys.append((y, expert_y))
+    torch.cuda.synchronize()
+    for ata in atas:
+        ata.destroy()
+
+    for rank in range(world_size):
+        rank_data = all_rank_data[rank // dp_size]
+        y = ys[rank][0]
+        ref_y = torch.zeros(rank_data.num_tokens, moe.hidden_dim, dtype=y.dtype, device=device)
+        for i_token in range(rank_data.num_tokens):
+            for i_expert in range(moe.experts_per_token):
+                weight = float(rank_data.weights[i_token, i_expert].item())
+                ref_y[i_token] += rank_data.x[i_token].to(device).to(y.dtype) * val * weight
+        torch.testing.assert_close(y[: rank_data.num_tokens], ref_y)
+        assert torch.isnan(y[rank_data.num_tokens :]).all()
+
+
+# ---------------------------------------------------------------------------
+# Committed golden vectors through the C ABI
+# ---------------------------------------------------------------------------
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+def test_golden_vectors(path):
+    z = np.load(path, allow_pickle=False)
+    E, K, H, M, G, R, esz, S, cap = (int(v) for v in z["meta"])
+    name = os.path.basename(path)
+    in_dtype = {"small_bf16": torch.bfloat16, "small_fp8": FP8, "small_f16": torch.float16}[name[:-4]]
+    out_dtype = torch.float16 if name.startswith("small_f16") else torch.bfloat16
+    dp = R // G
+    spec = WorkloadSpec(name, 0, R, E, K, H, M, in_dtype, out_dtype=out_dtype, expert_y_dtype=out_dtype, dp_size=dp)
+    groups = []
+    for g in range(G):
+        n = int(z[f"n_{g}"][0])
+        x = torch.from_numpy(z[f"x_{g}"].copy()).view(in_dtype).reshape(n, H)
+        xs = torch.from_numpy(z[f"x_scale_{g}"].copy()) if S else None
+        groups.append(
+            GroupInputs(x, xs, torch.from_numpy(z[f"indices_{g}"].astype(np.int32)), torch.from_numpy(z[f"weights_{g}"].copy()), n)
+        )
+    step = DeviceStep(spec, groups, cap=cap)
+    world = make_world(spec, group_name=name)
+    step.dispatch_world(world)
+    torch.cuda.synchronize()
+    L = E // R
+    counts = step.expert_num_tokens_all.cpu().numpy().reshape(E)
+    np.testing.assert_array_equal(counts, z["counts"])
+    live = np.arange(cap)[None, :] < counts[:, None]
+    got = step.expert_x_all.view(torch.uint8).reshape(E, cap, -1).cpu().numpy()
+    np.testing.assert_array_equal(got[live], z["expert_x"][live])
+    if S:
+        gs = step.expert_x_scale_all.reshape(E, cap, S).cpu().numpy()
+        np.testing.assert_array_equal(gs[live].view(np.uint32), z["expert_x_scale"][live].view(np.uint32))
+    y = torch.from_numpy(z["expert_y_bits"].view(np.int16).copy()).view(out_dtype).reshape(R, L, cap, H)
+    step.expert_y_all.copy_(y.cuda())
+    step.combine_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() == 0
+    world.destroy()
+    for r in range(R):
+        n = groups[r // dp].n
+        want = torch.from_numpy(z[f"out_{r // dp}"].view(np.int16).copy()).view(out_dtype).float()
+        got_y = step.out_tokens[r].cpu().float()
+        np.testing.assert_allclose(got_y[:n].numpy(), want.numpy(), rtol=COMBINE_RTOL, atol=COMBINE_ATOL)
+        assert torch.isnan(got_y[n:]).all()
+
+
+# ---------------------------------------------------------------------------
+# The benchmark workloads
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("api", ["world", "per_rank"])
+@pytest.mark.parametrize("cfg", ["C1", "C2", "C3"])
+def test_baseline_config_full_size(cfg, api):
+    spec = baseline_configs()[cfg]
+    run_and_check(spec, generate(spec), api=api)
+
+
+def test_c4_reduced_against_oracle():
+    spec = dataclasses.replace(baseline_configs()["C4"], max_num_tokens=640, hidden_dim=1024)
+    groups = generate(spec)
+    cap = int(expert_counts(groups, spec.num_experts).max())
+    run_and_check(spec, groups, cap=cap, use_numpy=True)
+
+
+def test_c5_reduced_against_oracle():
+    spec = dataclasses.replace(baseline_configs()["C5"], max_num_tokens=700, hidden_dim=1024)
+    groups = generate(spec)
+    cap = int(expert_counts(groups, spec.num_experts).max())
+    run_and_check(spec, groups, cap=cap, use_numpy=True)
+
+
+def _full_size_properties(cfg_name: str):
+    """Full-size check with properties that need no CPU pass over the payload: counts equal
+    a device bincount, every expert's rows equal the source rows in canonical order (a
+    device-side stable sort), and the reference's round-trip identity holds."""
+    spec = baseline_configs()[cfg_name]
+    groups = generate(spec)
+    counts = expert_counts(groups, spec.num_experts)
+    cap = int(counts.max())
+    step = DeviceStep(spec, groups, cap=cap)
+    world = make_world(spec, group_name=f"full-{cfg_name}")
+    step.dispatch_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() == 0
+    E, K, M, H = spec.num_experts, spec.experts_per_token, spec.max_num_tokens, spec.hidden_dim
+    np.testing.assert_array_equal(step.expert_num_tokens_all.cpu().numpy().reshape(E), counts)
+    dev = torch.device("cuda:0")
+    flat_e = torch.cat([g.indices[: g.n].reshape(-1) for g in groups]).to(dev).long()
+    tok_of_pair = torch.cat(
+        [torch.arange(g.n).repeat_interleave(K) + gi * M for gi, g in enumerate(groups)]
+    ).to(dev)
+    order = torch.argsort(flat_e, stable=True)
+    starts = torch.cumsum(torch.from_numpy(counts).to(dev), 0) - torch.from_numpy(counts).to(dev)
+    e_sorted = flat_e[order]
+    slot_sorted = torch.arange(order.numel(), device=dev) - starts[e_sorted]
+    src_tok = tok_of_pair[order]
+    all_x = torch.stack([g.x for g in groups]).to(dev).view(torch.uint8).reshape(len(groups) * M, -1)
+    got_x = step.expert_x_all.view(torch.uint8).reshape(E * cap, -1)
+    rows = e_sorted * cap + slot_sorted
+    chunk = 1 << 15
+    for i in range(0, rows.numel(), chunk):
+        assert torch.equal(got_x[rows[i : i + chunk]], all_x[src_tok[i : i + chunk]])
+    if spec.scale_dim:
+        all_s = torch.stack([g.x_scale for g in groups]).to(dev).reshape(len(groups) * M, -1)
+        got_s = step.expert_x_scale_all.reshape(E * cap, -1)
+        assert torch.equal(got_s[rows].view(torch.int32), all_s[src_tok].view(torch.int32))
+    # round trip (tests/test_all_to_all.py:249-250,277-286): y = sum_k w_k * 1.5 * x
+    for r in range(spec.world_size):
+        step.expert_y_all[r].copy_(step.expert_x_all[r].to(torch.bfloat16) * 1.5)
+    step.combine_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() == 0
+    world.destroy()
+    for r, g in enumerate(groups):
+        x = g.x[: g.n].to(dev).to(torch.float32) * 1.5
+        want = x * g.weights[: g.n].to(dev).sum(dim=1, keepdim=True)
+        got = step.out_tokens[r][: g.n].float()
+        torch.testing.assert_close(got, want, rtol=COMBINE_RTOL, atol=2 * COMBINE_ATOL)
+        assert torch.isnan(step.out_tokens[r][g.n :]).all()
+
+
+def test_c4_full_size_properties():
+    _full_size_properties("C4")
+
+
+def test_c5_full_size_properties():
+    _full_size_properties("C5")
+
+
+# ---------------------------------------------------------------------------
+# Edge cases
+# ---------------------------------------------------------------------------
+def _small_spec(**kw) -> WorkloadSpec:
+    base = dict(
+        name="edge", config_id=50, world_size=4, num_experts=16, experts_per_token=3,
+        hidden_dim=256, max_num_tokens=24, in_dtype=torch.bfloat16, tokens="uniform",
+    )  # fmt: skip
+    base.update(kw)
+    return WorkloadSpec(**base)
+
+
+@pytest.mark.parametrize("api", ["world", "per_rank"])
+def test_without_bound_m(api):
+    spec = _small_spec(name="nobound", tokens="max")
+    run_and_check(spec, generate(spec), api=api, with_bound_m=False)
+
+
+def test_empty_and_ragged_ranks():
+    spec = _small_spec(name="ragged", in_dtype=FP8, hidden_dim=512)
+    groups = generate(spec)
+    for g, n in zip(groups, [0, 24, 1, 7]):
+        g.n = n
+    run_and_check(spec, groups)
+    for g in groups:
+        g.n = 0
+    step = run_and_check(spec, groups)
+    assert int(step.expert_num_tokens_all.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dp_size", [2, 4])
+def test_dp_groups(dp_size):
+    spec = _small_spec(name=f"dp{dp_size}", dp_size=dp_size, in_dtype=FP8, hidden_dim=512)
+    run_and_check(spec, generate(spec), api="per_rank")
+
+
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_combine_dtype_matrix(y_dtype, out_dtype):
+    """The six (expert_y, out_tokens) pairs of csrc/bindings/all_to_all_ops.cpp:265-310."""
+    spec = _small_spec(name="dtypes", expert_y_dtype=y_dtype, out_dtype=out_dtype)
+    run_and_check(spec, generate(spec))
+
+
+@pytest.mark.parametrize(
+    "E,K,M,R",
+    [(512, 8, 300, 8), (1024, 4, 130, 4), (8, 8, 70, 2), (4, 1, 5, 1), (64, 6, 1500, 2), (2048, 2, 40, 2)],
+)
+def test_geometries(E, K, M, R):
+    """Expert counts that change the routing tile shape, several tiles, K = E, K = 1."""
+    spec = _small_spec(name=f"geo{E}", world_size=R, num_experts=E, experts_per_token=K, max_num_tokens=M, hidden_dim=128)
+    run_and_check(spec, generate(spec), use_numpy=True)
+
+
+@pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 16384 + 32, 40960])
+def test_row_sizes(hidden_bytes):
+    """Rows from one 16-byte vector up to the streaming path for rows beyond 32 KiB."""
+    spec = _small_spec(name=f"row{hidden_bytes}", hidden_dim=hidden_bytes // 2, max_num_tokens=9)
+    run_and_check(spec, generate(spec))
+
+
+def test_strided_scales():
+    """Scale tensors need not be contiguous (csrc/bindings/all_to_all_ops.cpp:137-146,174-179)."""
+    spec = _small_spec(name="strided", in_dtype=FP8, hidden_dim=1024)
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    R, L, S = spec.world_size, spec.num_local_experts, spec.scale_dim
+    # column-major scale inputs, and outputs laid out [L, S, cap] viewed as [L, cap, S]
+    step.dp_x_scale = [t.t().contiguous().t() for t in step.dp_x_scale]
+    backing = torch.zeros((R, L, S, step.cap), dtype=torch.float32, device="cuda")
+    step.expert_x_scale_all = backing.permute(0, 1, 3, 2)
+    step.expert_x_scale = [step.expert_x_scale_all[r] for r in range(R)]
+    assert not step.expert_x_scale[0].is_contiguous() and not step.dp_x_scale[0].is_contiguous()
+    world = make_world(spec, group_name="strided")
+    step.dispatch_world(world)
+    check_dispatch_against_oracle(step)
+    world.destroy()
+
+
+def test_row_capacity_overflow_is_reported_not_written():
+    spec = _small_spec(name="overflow", tokens="max")
+    groups = generate(spec)
+    counts = expert_counts(groups, spec.num_experts)
+    cap = int(counts.max()) - 2
+    step = DeviceStep(spec, groups, cap=cap)
+    guard = step.expert_x_all.clone().fill_(0)
+    step.expert_x_all.fill_(0)
+    world = make_world(spec, group_name="overflow")
+    step.dispatch_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() & 1
+    assert world.faults() == 0  # reading clears
+    # counts still report the full demand; rows that fit are in place
+    np.testing.assert_array_equal(step.expert_num_tokens_all.cpu().numpy().reshape(-1), counts)
+    from oracle import a2a_oracle as orc
+    from tests.all_to_all_utils import to_oracle_groups
+
+    full = orc.c_dispatch(to_oracle_groups(groups), spec.max_num_tokens, spec.num_experts, spec.experts_per_token, int(counts.max()))
+    got = step.expert_x_all.view(torch.uint8).reshape(spec.num_experts, cap, -1).cpu().numpy()
+    live = np.arange(cap)[None, :] < counts[:, None]
+    np.testing.assert_array_equal(got[live], full.expert_x[:, :cap][live])
+    del guard
+    world.destroy()
+
+
+def test_out_of_range_expert_is_ignored_and_reported():
+    spec = _small_spec(name="badidx", tokens="max")
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    step.indices[1] = step.indices[1].to(torch.int64).clone().index_fill_(0, torch.tensor([3], device="cuda"), 999).to(torch.uint32)
+    world = make_world(spec, group_name="badidx")
+    step.dispatch_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() & 2
+    total = int(step.expert_num_tokens_all.sum())
+    assert total == spec.experts_per_token * (sum(g.n for g in groups) - 1)
+    world.destroy()
+
+
+# ---------------------------------------------------------------------------
+# hipGraph replay (decode shape)
+# ---------------------------------------------------------------------------
+def test_graph_replay_decode_shape():
+    """C3: one captured dispatch+combine step replayed with changing inputs, routing and
+    bound_m; every replay is compared with the oracle, with eager work in between."""
+    spec = baseline_configs()["C3"]
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    world = make_world(spec, group_name="graph")
+    stream = torch.cuda.Stream()
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    step.expert_y_all.copy_(torch.randn(step.expert_y_all.shape, generator=gen, device="cuda"))
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        step.dispatch_world(world)  # warm-up outside capture
+        step.combine_world(world)
+        stream.synchronize()
+        with world.capture() as cap:
+            step.dispatch_world(world)
+            step.combine_world(world)
+        graph = cap.graph
+        for it in range(4):
+            new = generate(spec, seed=100 + it)
+            for r, g in enumerate(new):
+                if it % 2 == 1 and r % 3 == 0:
+                    g.n = 0
+                step.dp_x[r].copy_(g.x.cuda())
+                step.dp_x_scale[r].copy_(g.x_scale.cuda())
+                step.indices[r].copy_(g.indices.cuda().to(torch.uint32))
+                step.weights[r].copy_(g.weights.cuda())
+                step.bound_m[r].copy_(torch.tensor([g.n], dtype=torch.uint32).cuda())
+                step.out_tokens[r].fill_(float("nan"))
+            step.groups = new
+            stream.synchronize()
+            graph.replay(stream)
+            stream.synchronize()
+            expected = check_dispatch_against_oracle(step)
+            check_combine_against_oracle(step, expected.slot_map)
+            # eager work between replays
+            (step.expert_y_all.float().sum() + 1).item()
+        graph.destroy()
+    assert world.faults() == 0
+    world.destroy()
+
+
+# ---------------------------------------------------------------------------
+# Error behaviour
+# ---------------------------------------------------------------------------
+def test_errors_are_runtime_errors():
+    from pplx_kernels import AllToAll
+
+    spec = _small_spec(name="errors", tokens="max")
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    ranks = [
+        AllToAll.intranode(
+            spec.max_num_tokens, spec.num_experts, spec.experts_per_token, r, spec.world_size, 1,
+            spec.hidden_dim, spec.hidden_dim_bytes, 0, group_name="errors",
+        )  # fmt: skip
+        for r in range(spec.world_size)
+    ]
+    a = ranks[0]
+    kw = dict(
+        out_expert_num_tokens=step.expert_num_tokens[0], out_expert_x=step.expert_x[0], out_expert_x_scale=None,
+        dp_x=step.dp_x[0], dp_x_scale=None, indices=step.indices[0], bound_m=step.bound_m[0],
+    )  # fmt: skip
+    with pytest.raises(RuntimeError, match="Invalid split mode"):
+        a.dispatch(**kw, do_send=False, do_recv=False)
+    with pytest.raises(RuntimeError, match="indices must be of type UInt32"):
+        a.dispatch(**{**kw, "indices": step.indices[0].to(torch.int32)})
+    with pytest.raises(RuntimeError, match="must be on GPU"):
+        a.dispatch(**{**kw, "dp_x": step.dp_x[0].cpu()})
+    with pytest.raises(RuntimeError, match="experts per token"):
+        a.dispatch(**{**kw, "indices": step.indices[0][:, :2].contiguous()})
+    with pytest.raises(RuntimeError, match="boundM must be a scalar tensor"):
+        a.dispatch(**{**kw, "bound_m": torch.zeros(2, dtype=torch.uint32, device="cuda")})
+    a.dispatch(**kw)
+    with pytest.raises(RuntimeError, match="twice"):
+        a.dispatch(**kw)
+    with pytest.raises(RuntimeError, match="Unsupported dtype for outTokens"):
+        a.combine(
+            out_tokens=step.out_tokens[0].float(), indices=step.indices[0], weights=step.weights[0],
+            expert_y=step.expert_y[0], bound_m=None,
+        )  # fmt: skip
+    # finish the step so that the world is left consistent
+    for r in range(1, spec.world_size):
+        step_kw = dict(
+            out_expert_num_tokens=step.expert_num_tokens[r], out_expert_x=step.expert_x[r], out_expert_x_scale=None,
+            dp_x=step.dp_x[r], dp_x_scale=None, indices=step.indices[r], bound_m=step.bound_m[r],
+        )  # fmt: skip
+        ranks[r].dispatch(**step_kw)
+    check_dispatch_against_oracle(step)
+    for r in ranks:
+        r.destroy()
+    ranks[0].destroy()  # idempotent
