@@ -132,7 +132,10 @@ int check_config(const pplx_a2a_config_t &c) {
   const uint64_t groups = c.world_size / c.dp_size;
   if (groups * c.max_num_tokens > (1ull << 30) ||
       groups * c.max_num_tokens * c.experts_per_token > (1ull << 31) ||
-      c.hidden_dim_bytes > (1ull << 30) || c.num_experts > 5461)
+      c.hidden_dim_bytes > (1ull << 30) || c.num_experts > 5461 ||
+      // one wave per (rank, token, 512-element segment) / per (token, pick share): 32-bit grids
+      (uint64_t)c.world_size * c.max_num_tokens * ((c.hidden_dim + 511) / 512) > (1ull << 32) ||
+      groups * c.max_num_tokens * 64 > (1ull << 32))
     return fail(PPLX_A2A_UNSUPPORTED, "geometry exceeds the limits of this build");
   return PPLX_A2A_OK;
 }

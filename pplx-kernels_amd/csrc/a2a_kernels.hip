@@ -14,8 +14,8 @@
 //                    is read once into registers and stored K times, 16 B / lane
 //   dispatch_fused   small steps: routing and scatter in one launch; every
 //                    workgroup recounts the picks of the tokens before its own
-//   combine_gather   one workgroup per token: K rows gathered through the slot
-//                    map, fp32 accumulate in pick order, 16 B stores
+//   combine_gather   one wave per 1 KiB of an output row: K rows gathered through
+//                    the slot map, fp32 accumulate in pick order, 16 B stores
 //
 // No atomics on global memory (fault flags aside), no spin waits, no
 // cooperative launch: phase boundaries are kernel boundaries on one stream, so a
@@ -52,6 +52,58 @@ struct InlineCombine {
 struct HbmCombine {
   const CombineRank *rows;
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
+};
+
+// Pointers rebuilt from integers would be "flat" to the compiler; these casts say
+// that they are global memory, so that plain global_load / global_store are emitted.
+#define PPLX_GLOBAL __attribute__((address_space(1)))
+template <typename V>
+__device__ __forceinline__ PPLX_GLOBAL V *global_ptr(uint64_t address) {
+  return (PPLX_GLOBAL V *)address;
+}
+template <typename V>
+__device__ __forceinline__ const PPLX_GLOBAL V *global_cptr(uint64_t address) {
+  return (const PPLX_GLOBAL V *)address;
+}
+
+// Makes the compiler treat `v` as consumed here, so that it waits for the loads
+// feeding it at this point and not inside a later loop, where such a wait would
+// also drain the stores of the previous iteration.
+template <typename V>
+__device__ __forceinline__ void settle(V &v) {
+  asm volatile("" : "+v"(v));
+}
+
+// settle() for N registers at once: every load feeding them has to be issued
+// before this point, so the N loads go out back to back behind one wait.
+template <int N> struct SettleAll;
+template <> struct SettleAll<1> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) { asm volatile("" : "+v"(r[0])); }
+};
+template <> struct SettleAll<2> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]));
+  }
+};
+template <> struct SettleAll<4> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+  }
+};
+template <> struct SettleAll<8> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile(""
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
+                   "+v"(r[7]));
+  }
+};
+template <> struct SettleAll<16> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile(""
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
+                   "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]),
+                   "+v"(r[13]), "+v"(r[14]), "+v"(r[15]));
+  }
 };
 
 __device__ __forceinline__ uint32_t lane_id() {
@@ -236,19 +288,26 @@ __device__ __forceinline__ void fan_out_row(const WorldDev &w, const DT &tab, ui
     }
   }
 
+#pragma unroll
+  for (int i = 0; i < NV; ++i) settle(x[i]);
+  settle(sc);
+  settle(dst_row);
+  settle(dst_scale);
+  settle(dst_scale_step);
+
   for (uint32_t k = k0; k < k1; ++k) {
     const uint64_t p = read_lane64(dst_row, k);
     if (p == 0) continue;
-    u32x4 *out = reinterpret_cast<u32x4 *>(p);
+    PPLX_GLOBAL u32x4 *out = global_ptr<u32x4>(p);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const uint32_t j = lane + i * kWave;
       if (EXACT || j < nvec) __builtin_nontemporal_store(x[i], out + j);
     }
     if (S) {
-      float *sout = reinterpret_cast<float *>(read_lane64(dst_scale, k));
+      PPLX_GLOBAL float *sout = global_ptr<float>(read_lane64(dst_scale, k));
       const int64_t step = (int64_t)read_lane64((uint64_t)dst_scale_step, k);
-      if (lane < S) sout[(int64_t)lane * step] = sc;
+      if (lane < S) __builtin_nontemporal_store(sc, sout + (int64_t)lane * step);
       for (uint32_t j = lane + kWave; j < S; j += kWave) {
         sout[(int64_t)j * step] = srow[(int64_t)j * src.dp_xs_stride_elem];
       }
@@ -280,7 +339,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
 // order, then fans the rows out.  The last workgroup has counted everything
 // and writes out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+__global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
   extern __shared__ uint32_t lds_u32[];
   uint32_t *hist = lds_u32;             // [E]
   uint32_t *ntok = hist + w.E;          // [G]
@@ -419,17 +478,21 @@ template <> struct Row8<float> {
     f32x4 a, b;
   };
   static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
-    const f32x4 *p = reinterpret_cast<const f32x4 *>(row) + 2 * (size_t)vec;
+    const PPLX_GLOBAL f32x4 *p = global_cptr<f32x4>(row) + 2 * (size_t)vec;
     return Raw{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1)};
   }
   static __device__ __forceinline__ f32x8 widen(const Raw &r) {
     return __builtin_shufflevector(r.a, r.b, 0, 1, 2, 3, 4, 5, 6, 7);
   }
+  // N rows held as 2 N registers of 16 bytes
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) {
+    SettleAll<2 * N>::of(reinterpret_cast<f32x4 *>(raw));
+  }
 };
 template <> struct Row8<__bf16> {
   typedef u32x4 Raw;
   static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + vec);
+    return __builtin_nontemporal_load(global_cptr<u32x4>(row) + vec);
   }
   static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
     f32x8 out;
@@ -440,26 +503,28 @@ template <> struct Row8<__bf16> {
     }
     return out;
   }
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) { SettleAll<N>::of(raw); }
 };
 template <> struct Row8<_Float16> {
   typedef f16x8 Raw;
   static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
-    return __builtin_nontemporal_load(reinterpret_cast<const f16x8 *>(row) + vec);
+    return __builtin_nontemporal_load(global_cptr<f16x8>(row) + vec);
   }
   static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
     return __builtin_convertvector(raw, f32x8);
   }
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) { SettleAll<N>::of(raw); }
 };
 
 template <typename U> struct Store8;
 template <> struct Store8<__bf16> {
   static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
-    reinterpret_cast<bf16x8 *>(row)[vec] = __builtin_convertvector(acc, bf16x8);
+    __builtin_nontemporal_store(__builtin_convertvector(acc, bf16x8), reinterpret_cast<bf16x8 *>(row) + vec);
   }
 };
 template <> struct Store8<_Float16> {
   static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
-    reinterpret_cast<f16x8 *>(row)[vec] = __builtin_convertvector(acc, f16x8);
+    __builtin_nontemporal_store(__builtin_convertvector(acc, f16x8), reinterpret_cast<f16x8 *>(row) + vec);
   }
 };
 
@@ -470,6 +535,7 @@ __device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, f
   typename Row8<T>::Raw raw[N];
 #pragma unroll
   for (int i = 0; i < N; ++i) raw[i] = Row8<T>::load(read_lane64(row_of_lane, k + i), vec);
+  Row8<T>::template settle<N>(raw);
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     const float wk = __builtin_bit_cast(
@@ -478,15 +544,24 @@ __device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, f
   }
 }
 
-template <typename T, typename U, class CT>
-__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab) {
-  const uint32_t r = blockIdx.x / w.M;
-  const uint32_t t = blockIdx.x - r * w.M;
+// One wave owns VPL * 64 consecutive 8-element vectors of one output row.  With
+// KK == 0 (any K) it is one vector per lane and the picks go in groups of up to
+// eight loads; with KK in {1, 2, 4} the wave takes VPL = 8 / KK vectors per lane so
+// that eight row loads per lane are in flight for small top-k too.
+template <typename T, typename U, class CT, int KK, int VPL>
+__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments) {
+  const uint32_t lane = lane_id();
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
+                                                       threadIdx.x / kWave);
+  const uint32_t token = wave / segments;
+  const uint32_t segment = wave - token * segments;
+  const uint32_t r = token / w.M;
+  const uint32_t t = token - r * w.M;
+  if (r >= w.R) return;
   const CombineRank &c = tab.at(r);
   if (t >= combine_rank_tokens(w, c)) return;
 
-  // Every wave resolves the K picks itself (lane k <-> pick k): no LDS, no barrier.
-  const uint32_t lane = lane_id();
+  // Lane k resolves pick k: no LDS, no barrier.
   uint64_t row = 0;
   float weight = 0.f;
   if (lane < w.K) {
@@ -499,7 +574,7 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab) {
         row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
                                          (int64_t)(e % w.L) * owner.y_stride_expert +
                                          (int64_t)slot * owner.y_stride_row);
-      } else if (threadIdx.x == lane) {
+      } else if (segment == 0) {
         atomicOr(w.faults, kFaultBadSlot);
       }
     }
@@ -509,24 +584,51 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab) {
   U *out = reinterpret_cast<U *>(c.out_tokens) + (int64_t)t * c.out_stride_row;
   const uint32_t nvec = w.H / 8;
   const uint32_t K = w.K;
-  if (all_rows) {
-    for (uint32_t vec = threadIdx.x; vec < nvec; vec += blockDim.x) {
-      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      uint32_t k = 0;
-      for (; k + 8 <= K; k += 8) gather_group<T, 8>(acc, row, weight, k, vec);
-      if (K & 4) { gather_group<T, 4>(acc, row, weight, k, vec); k += 4; }
-      if (K & 2) { gather_group<T, 2>(acc, row, weight, k, vec); k += 2; }
-      if (K & 1) { gather_group<T, 1>(acc, row, weight, k, vec); }
-      Store8<U>::at(out, vec, acc);
-    }
-  } else {
+  if (!all_rows) {
     // A pick without a row (bad expert id or slot) contributes nothing.
-    for (uint32_t vec = threadIdx.x; vec < nvec; vec += blockDim.x) {
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
       f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       for (uint32_t k = 0; k < K; ++k) {
-        if (read_lane64(row, k) != 0) gather_group<T, 1>(acc, row, weight, k, vec);
+        if (read_lane64(row, k) != 0) gather_group<T, 1>(acc, row, weight, k, vec_ld);
       }
-      Store8<U>::at(out, vec, acc);
+      if (vec < nvec) Store8<U>::at(out, vec, acc);
+    }
+    return;
+  }
+  if (KK == 0) {
+    const uint32_t vec = segment * kWave + lane;
+    const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;  // clamp: loads stay unconditional
+    f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint32_t k = 0;
+    for (; k + 8 <= K; k += 8) gather_group<T, 8>(acc, row, weight, k, vec_ld);
+    if (K & 4) { gather_group<T, 4>(acc, row, weight, k, vec_ld); k += 4; }
+    if (K & 2) { gather_group<T, 2>(acc, row, weight, k, vec_ld); k += 2; }
+    if (K & 1) { gather_group<T, 1>(acc, row, weight, k, vec_ld); }
+    if (vec < nvec) Store8<U>::at(out, vec, acc);
+  } else {
+    constexpr int N = KK == 0 ? 1 : KK;
+    typename Row8<T>::Raw raw[VPL][N];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
+#pragma unroll
+      for (int k = 0; k < N; ++k) raw[v][k] = Row8<T>::load(read_lane64(row, k), vec_ld);
+    }
+    Row8<T>::template settle<VPL * N>(&raw[0][0]);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        const float wk = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), k));
+        acc += wk * Row8<T>::widen(raw[v][k]);
+      }
+      if (vec < nvec) Store8<U>::at(out, vec, acc);
     }
   }
 }
@@ -560,6 +662,7 @@ int launch_route_t(const WorldDev &w, const DT &tab, hipStream_t s) {
 }
 
 // Picks the register variant for the row size and launches KERNEL<NV, EXACT, DT>.
+// Rows beyond 8 KiB exist only for dispatch_scatter (PPLX_LAUNCH_LARGE_ROW_VARIANT).
 #define PPLX_LAUNCH_ROW_VARIANT(KERNEL, NV, EXACT)                                               \
   hipLaunchKernelGGL((KERNEL<NV, EXACT, DT>), grid, block, lds, s, w, tab, ksplit, kper)
 
@@ -580,8 +683,7 @@ int launch_route_t(const WorldDev &w, const DT &tab, hipStream_t s) {
     else if (per_lane <= 2) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 2, false);                           \
     else if (per_lane <= 4) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 4, false);                           \
     else if (per_lane <= 8) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 8, false);                           \
-    else if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                         \
-    else PPLX_LAUNCH_ROW_VARIANT(KERNEL, 32, false);                                             \
+    else PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL);                                                  \
   } while (0)
 
 // Number of waves a row's K copies are spread over: few tokens -> more waves,
@@ -605,19 +707,28 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint64_t waves = (uint64_t)tokens * ksplit;
   const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
   const uint32_t lds = 0;
+#define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL)                                                    \
+  do {                                                                                           \
+    if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                              \
+    else PPLX_LAUNCH_ROW_VARIANT(KERNEL, 32, false);                                             \
+  } while (0)
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
+#undef PPLX_LAUNCH_LARGE_ROW_VARIANT
   return (int)hipGetLastError();
 }
 
 template <class DT>
 int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
-  const uint32_t ksplit = pick_ksplit(w, 4);  // 4 waves per workgroup
+  constexpr uint32_t kWaves = 16;  // 1024 threads: fewer, larger workgroups repeat less counting
+  const uint32_t ksplit = pick_ksplit(w, kWaves);
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
-  const uint32_t tokens_per_block = 4 / ksplit;
-  const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(256);
+  const uint32_t tokens_per_block = kWaves / ksplit;
+  const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
   const uint32_t lds = (w.E + w.G + tokens_per_block * w.K) * sizeof(uint32_t);
+#define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
+#undef PPLX_LAUNCH_LARGE_ROW_VARIANT
   return (int)hipGetLastError();
 }
 
@@ -629,20 +740,34 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   return launch_scatter_t(w, tab, s);
 }
 
-template <class CT>
-int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s) {
-  const dim3 grid(w.R * w.M), block(256);
-  // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
-  switch (in_dtype * 4 + out_dtype) {
-    case 0 * 4 + 1: hipLaunchKernelGGL((combine_gather<float, __bf16, CT>), grid, block, 0, s, w, tab); break;
-    case 0 * 4 + 2: hipLaunchKernelGGL((combine_gather<float, _Float16, CT>), grid, block, 0, s, w, tab); break;
-    case 1 * 4 + 1: hipLaunchKernelGGL((combine_gather<__bf16, __bf16, CT>), grid, block, 0, s, w, tab); break;
-    case 1 * 4 + 2: hipLaunchKernelGGL((combine_gather<__bf16, _Float16, CT>), grid, block, 0, s, w, tab); break;
-    case 2 * 4 + 1: hipLaunchKernelGGL((combine_gather<_Float16, __bf16, CT>), grid, block, 0, s, w, tab); break;
-    case 2 * 4 + 2: hipLaunchKernelGGL((combine_gather<_Float16, _Float16, CT>), grid, block, 0, s, w, tab); break;
-    default: return (int)hipErrorInvalidValue;
+template <typename T, typename U, class CT>
+int launch_combine_k(const WorldDev &w, const CT &tab, hipStream_t s) {
+  const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
+  const uint32_t vpl = w.K == 1 ? 8 : w.K == 2 ? 4 : w.K == 4 ? 2 : 1;
+  const uint32_t segments = (nvec_segments + vpl - 1) / vpl;
+  const uint64_t waves = (uint64_t)w.R * w.M * segments;
+  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
+  switch (w.K) {
+    case 1: hipLaunchKernelGGL((combine_gather<T, U, CT, 1, 8>), grid, block, 0, s, w, tab, segments); break;
+    case 2: hipLaunchKernelGGL((combine_gather<T, U, CT, 2, 4>), grid, block, 0, s, w, tab, segments); break;
+    case 4: hipLaunchKernelGGL((combine_gather<T, U, CT, 4, 2>), grid, block, 0, s, w, tab, segments); break;
+    default: hipLaunchKernelGGL((combine_gather<T, U, CT, 0, 1>), grid, block, 0, s, w, tab, segments); break;
   }
   return (int)hipGetLastError();
+}
+
+template <class CT>
+int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s) {
+  // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
+  switch (in_dtype * 4 + out_dtype) {
+    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, s);
+    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, s);
+    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, s);
+    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, s);
+    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, s);
+    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, s);
+    default: return (int)hipErrorInvalidValue;
+  }
 }
 
 }  // namespace
@@ -659,7 +784,7 @@ bool dispatch_is_fused(const WorldDev &w) {
   // while the whole step's routing is a few tens of KiB.
   const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
   const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
-  return pairs <= kFusedMaxPairs && per_lane <= 32 && (w.E + w.G + 4 * w.K) * 4 <= 48 * 1024;
+  return pairs <= kFusedMaxPairs && per_lane <= 8 && (w.E + w.G + 16 * w.K) * 4 <= 48 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {

@@ -1,0 +1,147 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads, exports every symbol
+that ``include/pplx_a2a.h`` declares, validates configurations without a GPU, and the
+Python binding layer raises the reference's errors before anything reaches the device.
+No compute call is made here."""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from pplx_kernels import AllToAll, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pplx_a2a.h")
+
+
+def declared_symbols() -> list[str]:
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pplx_a2a_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ops.load_library()
+    names = declared_symbols()
+    assert len(names) >= 17
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/pplx_a2a.h but not exported"
+    assert sorted(ops.EXPORTED_SYMBOLS) == names
+    assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.pplx_a2a_version())
+
+
+def test_ctypes_structs_match_the_header_layout():
+    # 8-byte fields throughout, except the trailing (u32 m) and the i32 dtypes, which pad to 8.
+    assert ctypes.sizeof(ops.Config) == 56
+    assert ctypes.sizeof(ops.DispatchArgs) == 18 * 8
+    assert ctypes.sizeof(ops.CombineArgs) == 12 * 8
+    assert ops.DispatchArgs.bound_m.offset == 17 * 8
+    assert ops.CombineArgs.in_dtype.offset == 10 * 8 and ops.CombineArgs.m.offset == 10 * 8 + 4
+
+
+def _create(cfg: tuple) -> tuple[int, str]:
+    lib = ops.load_library()
+    c = ops.Config(*cfg)
+    out = ctypes.c_void_p()
+    st = lib.pplx_a2a_world_create(ctypes.byref(c), 0, ctypes.byref(out))
+    return st, lib.pplx_a2a_last_error().decode()
+
+
+# (max_num_tokens, num_experts, experts_per_token, world_size, dp_size, hidden_dim, bytes, scale bytes)
+GOOD = (128, 256, 8, 8, 1, 7168, 7168, 224)
+
+
+@pytest.mark.parametrize(
+    "field,value,message",
+    [
+        (6, 7160, "invalid hidden dim bytes"),  # not a multiple of 16 (all_to_all.cpp:32)
+        (7, 220, "invalid hidden dim scale bytes"),  # (all_to_all.cpp:33)
+        (7, 7168 + 16, "invalid hidden dim bytes"),  # scale bytes > row bytes (all_to_all.cpp:39)
+        (4, 3, "multiple of dp_size"),
+        (1, 100, "multiple of world_size"),
+        (2, 0, "experts_per_token"),
+        (2, 65, "experts_per_token"),
+        (0, 0, "max_num_tokens"),
+        (3, 0, "world_size"),
+    ],
+)
+def test_world_create_rejects_bad_configs(field, value, message):
+    cfg = list(GOOD)
+    cfg[field] = value
+    st, err = _create(tuple(cfg))
+    assert st == 1, (st, err)
+    assert message in err
+
+
+def test_world_create_needs_a_gpu_for_good_configs():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    st, err = _create(GOOD)
+    assert st == 3 and "hip" in err.lower()  # HIP error, not a silent fallback
+    with pytest.raises(RuntimeError, match="HIP error"):
+        AllToAll.intranode(128, 256, 8, 0, 8, 1, 7168, 7168, 224)
+
+
+def test_null_arguments_are_status_codes_not_crashes():
+    lib = ops.load_library()
+    assert lib.pplx_a2a_world_create(None, 0, None) == 1
+    assert lib.pplx_a2a_create(None, 0, None) == 1
+    assert lib.pplx_a2a_dispatch(None, None, 0, None) == 1
+    assert lib.pplx_a2a_combine(None, None, 0, None) == 1
+    assert lib.pplx_a2a_world_dispatch(None, None, None) == 1
+    assert lib.pplx_a2a_world_faults(None, None, None) == 1
+    assert lib.pplx_a2a_graph_launch(None, None) == 1
+    assert lib.pplx_a2a_destroy(None) == 0 and lib.pplx_a2a_world_destroy(None) == 0
+    assert lib.pplx_a2a_graph_destroy(None) == 0
+
+
+def test_binding_checks_fire_before_the_device():
+    """The tensor checks of csrc/bindings/all_to_all_ops.cpp:135-161,249-259 run on CPU tensors."""
+    n, k, h = 4, 2, 64
+    i32 = torch.zeros(2, dtype=torch.int32)
+    x3 = torch.zeros(2, 8, h, dtype=torch.bfloat16)
+    x2 = torch.zeros(n, h, dtype=torch.bfloat16)
+    idx = torch.zeros(n, k, dtype=torch.uint32)
+    with pytest.raises(RuntimeError, match="Tensor outExpertNumTokens must be on GPU"):
+        ops.pack_dispatch_args(k, i32, x3, None, x2, None, idx, None)
+    with pytest.raises(RuntimeError, match="Tensor outTokens must be on GPU"):
+        ops.pack_combine_args(x2, idx, torch.zeros(n, k), x3, None)
+    with pytest.raises(RuntimeError, match="Invalid split mode"):
+        ops.split_mode(False, False)
+    assert (ops.split_mode(True, True), ops.split_mode(True, False), ops.split_mode(False, True)) == (0, 1, 2)
+
+
+def test_op_schemas_match_the_reference():
+    """csrc/bindings/all_to_all_ops.cpp:329-391: names, mutability and argument order."""
+    for transport in ("intranode", "internode"):
+        d = getattr(torch.ops.pplx_kernels, f"all_to_all_{transport}_dispatch").default._schema
+        assert [a.name for a in d.arguments] == [
+            "fptr", "out_expert_num_tokens", "out_expert_x", "out_expert_x_scale", "dp_x",
+            "dp_x_scale", "indices", "bound_m", "do_send", "do_recv",
+        ]  # fmt: skip
+        assert [a.name for a in d.arguments if a.alias_info and a.alias_info.is_write] == [
+            "out_expert_num_tokens", "out_expert_x", "out_expert_x_scale",
+        ]  # fmt: skip
+        c = getattr(torch.ops.pplx_kernels, f"all_to_all_{transport}_combine").default._schema
+        assert [a.name for a in c.arguments] == [
+            "fptr", "out_tokens", "indices", "weights", "expert_y", "bound_m", "do_send", "do_recv",
+        ]  # fmt: skip
+        assert [a.name for a in c.arguments if a.alias_info and a.alias_info.is_write] == ["out_tokens"]
+    assert hasattr(torch.ops.pplx_kernels, "all_to_all_destroy")
+    assert hasattr(torch.ops.pplx_kernels, "all_to_all_intranode_create")
+    assert hasattr(torch.ops.pplx_kernels, "all_to_all_internode_create")
+
+
+def test_meta_kernels_are_no_ops():
+    """Fake implementations let torch.compile trace the ops (all_to_all_ops.cpp:198-209,313-322)."""
+    m = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="meta")  # noqa: E731
+    torch.ops.pplx_kernels.all_to_all_intranode_dispatch(
+        0, m(2, dt=torch.int32), m(2, 8, 64), None, m(4, 64), None, m(4, 2, dt=torch.uint32), None, True, True
+    )
+    torch.ops.pplx_kernels.all_to_all_intranode_combine(
+        0, m(4, 64), m(4, 2, dt=torch.uint32), m(4, 2, dt=torch.float32), m(2, 8, 64), None, True, True
+    )
