@@ -185,6 +185,30 @@ def cpu_baseline(spec, groups, budget_s=20.0):
     }
 
 
+def counter_probe(spec, launches=3):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a few eager dispatch and
+    combine launches of the workload plus a plain elementwise copy of known size (1 GiB read,
+    1 GiB written) whose counter reading calibrates the unit."""
+    from tests.all_to_all_utils import DeviceStep, expert_counts, generate, make_world
+
+    groups = generate(spec)
+    cap = max(int(expert_counts(groups, spec.num_experts).max()), 1)
+    step = DeviceStep(spec, groups, cap=cap)
+    step.expert_y_all.normal_()
+    world = make_world(spec, group_name="probe")
+    a = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
+    b = torch.empty_like(a)
+    torch.cuda.synchronize()
+    for _ in range(launches):
+        torch.mul(a, 3, out=b)  # calibration: reads 2^30 bytes, writes 2^30 bytes
+        step.dispatch_world(world)
+        step.combine_world(world)
+        torch.cuda.synchronize()
+    d, c = step.algorithmic_bytes()
+    print(json.dumps({"probe": spec.name, "dispatch_bytes": d, "combine_bytes": c, "copy_bytes_each_way": 1 << 30}))
+    world.destroy()
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -193,6 +217,7 @@ def main() -> None:
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--all", action="store_true", help="also measure C1, C3, C4, C5 (reported under 'other_workloads')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--counter-probe", action="store_true", help="few eager launches + a calibration copy, for rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(
@@ -211,6 +236,9 @@ def main() -> None:
     ops.load_library()  # fail loudly here if the HIP library is missing
     specs = baseline_configs()
     spec = specs[args.workload]
+    if args.counter_probe:
+        counter_probe(spec)
+        return
     main_res, groups, steps = measure_workload(args.workload, spec, args.steps, args.warmup)
 
     # Roofline of the dominant kernel: graphs holding back-to-back combine_gather launches

@@ -95,6 +95,14 @@ struct pplx_a2a_world {
   bool captured_once = false;
   // Capture session that recorded the last bind of each table (0 = an eager bind).
   unsigned long long bind_capture_dispatch = 0, bind_capture_combine = 0;
+
+  // Split send / recv mode: staging is allocated by the first split call; the masks record
+  // which ranks have made which call of the step in flight.
+  SplitDev split{};
+  bool split_ready = false;
+  std::vector<uint8_t> dsend, drecv, csend, crecv;
+  uint32_t n_dsend = 0, n_drecv = 0, n_csend = 0, n_crecv = 0;
+  int split_in_dtype = -1;
 };
 
 struct pplx_a2a {
@@ -306,6 +314,166 @@ int run_combine(pplx_a2a_world &w, void *stream) {
   return PPLX_A2A_OK;
 }
 
+uint64_t round_up(uint64_t x, uint64_t to) { return (x + to - 1) / to * to; }
+
+void free_split(pplx_a2a_world &w) {
+  SplitDev &sp = w.split;
+  (void)hipFree(sp.stage_x);
+  (void)hipFree(sp.gtile_cnt);
+  (void)hipFree(sp.gslot);
+  (void)hipFree(sp.gexp);
+  (void)hipFree(sp.gcnt);
+  (void)hipFree(sp.goff);
+  (void)hipFree(sp.gbase);
+  (void)hipFree(sp.gntok);
+  (void)hipFree(sp.stage_y);
+  sp = SplitDev{};
+  w.split_ready = false;
+}
+
+// Allocates the staging of split mode on first use (never inside a stream capture).
+int ensure_split(pplx_a2a_world &w, void *stream) {
+  if (w.split_ready) return PPLX_A2A_OK;
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
+  if (st) return st;
+  if (session != 0)
+    return fail(PPLX_A2A_INVALID_STATE,
+                "the first split send/recv call allocates staging and cannot be captured; "
+                "run one eager step first");
+  const WorldDev &d = w.dev;
+  SplitDev &sp = w.split;
+  sp.token_stride = (uint32_t)round_up((uint64_t)d.Hb + 4ull * d.S + 4, 16);
+  const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
+  sp.tiles_per_group = (uint32_t)((d.M + tile_tokens - 1) / tile_tokens);
+  const size_t pairs = (size_t)d.G * d.M * d.K;
+  struct Alloc {
+    void **ptr;
+    size_t bytes;
+  } allocs[] = {
+      {reinterpret_cast<void **>(&sp.stage_x), pairs * sp.token_stride},
+      {reinterpret_cast<void **>(&sp.gtile_cnt), sizeof(uint32_t) * (size_t)d.G * sp.tiles_per_group * d.E},
+      {reinterpret_cast<void **>(&sp.gslot), sizeof(uint32_t) * pairs},
+      {reinterpret_cast<void **>(&sp.gexp), sizeof(uint32_t) * pairs},
+      {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.G * d.E},
+      {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.G * d.E},
+      {reinterpret_cast<void **>(&sp.gbase), sizeof(uint32_t) * (size_t)d.G * d.E},
+      {reinterpret_cast<void **>(&sp.gntok), sizeof(uint32_t) * (size_t)d.G},
+  };
+  for (const Alloc &a : allocs) {
+    hipError_t err = hipMalloc(a.ptr, a.bytes);
+    if (err == hipSuccess) err = hipMemset(*a.ptr, 0, a.bytes);
+    if (err != hipSuccess) {
+      free_split(w);
+      return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of split-mode staging failed: %s", a.bytes,
+                  hipGetErrorString(err));
+    }
+  }
+  w.dsend.assign(d.R, 0);
+  w.drecv.assign(d.R, 0);
+  w.csend.assign(d.R, 0);
+  w.crecv.assign(d.R, 0);
+  w.split_ready = true;
+  return PPLX_A2A_OK;
+}
+
+// stage_y holds one expert_y row per (token, pick); sized for the widest dtype seen so far.
+int ensure_stage_y(pplx_a2a_world &w, int in_dtype, void *stream) {
+  const uint64_t row_bytes = (uint64_t)w.dev.H * dtype_size(in_dtype);
+  SplitDev &sp = w.split;
+  if (sp.stage_y && sp.y_row_bytes == row_bytes) return PPLX_A2A_OK;
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
+  if (st) return st;
+  if (session != 0)
+    return fail(PPLX_A2A_INVALID_STATE,
+                "the first split combine of a dtype allocates staging and cannot be captured");
+  HIP_TRY(hipDeviceSynchronize());
+  (void)hipFree(sp.stage_y);
+  sp.stage_y = nullptr;
+  const size_t bytes = (size_t)w.dev.G * w.dev.M * w.dev.K * row_bytes;
+  hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_y), bytes);
+  if (err != hipSuccess)
+    return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of combine staging failed: %s", bytes,
+                hipGetErrorString(err));
+  sp.y_row_bytes = row_bytes;
+  return PPLX_A2A_OK;
+}
+
+int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, int mode, void *stream) {
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  if (w.n_arrived_dispatch != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a send+recv dispatch step is still being assembled");
+  int st = ensure_split(w, stream);
+  if (st) return st;
+  const uint32_t R = w.dev.R;
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    if (w.n_drecv != 0)
+      return fail(PPLX_A2A_INVALID_STATE,
+                  "rank %u: dispatch SEND of the next step before every rank's RECV of this one", rank);
+    if (w.dsend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called dispatch SEND twice", rank);
+    LAUNCH_TRY(launch_split_dispatch_send(w.dev, w.split, row, rank, stream));
+    w.dsend[rank] = 1;
+    ++w.n_dsend;
+    return PPLX_A2A_OK;
+  }
+  if (w.n_dsend != R)
+    return fail(PPLX_A2A_INVALID_STATE,
+                "rank %u: dispatch RECV before every rank's SEND (%u of %u sent); in a loopback "
+                "world all SENDs must be enqueued first", rank, w.n_dsend, R);
+  if (w.drecv[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called dispatch RECV twice", rank);
+  LAUNCH_TRY(launch_split_dispatch_recv(w.dev, w.split, row, rank, w.n_drecv == 0, stream));
+  w.drecv[rank] = 1;
+  if (++w.n_drecv == R) {
+    std::fill(w.dsend.begin(), w.dsend.end(), 0);
+    std::fill(w.drecv.begin(), w.drecv.end(), 0);
+    w.n_dsend = w.n_drecv = 0;
+  }
+  return PPLX_A2A_OK;
+}
+
+int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int in_dtype, int out_dtype,
+                  int mode, void *stream) {
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  if (w.n_arrived_combine != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a send+recv combine step is still being assembled");
+  int st = ensure_split(w, stream);
+  if (st) return st;
+  const uint32_t R = w.dev.R;
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    if (w.n_crecv != 0)
+      return fail(PPLX_A2A_INVALID_STATE,
+                  "rank %u: combine SEND of the next step before every rank's RECV of this one", rank);
+    if (w.csend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine SEND twice", rank);
+    if (w.n_csend != 0 && w.split_in_dtype != in_dtype)
+      return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
+    st = ensure_stage_y(w, in_dtype, stream);
+    if (st) return st;
+    w.split_in_dtype = in_dtype;
+    LAUNCH_TRY(launch_split_combine_send(w.dev, w.split, row, rank, in_dtype, stream));
+    w.csend[rank] = 1;
+    ++w.n_csend;
+    return PPLX_A2A_OK;
+  }
+  if (w.n_csend != R)
+    return fail(PPLX_A2A_INVALID_STATE,
+                "rank %u: combine RECV before every rank's SEND (%u of %u sent); in a loopback "
+                "world all SENDs must be enqueued first", rank, w.n_csend, R);
+  if (w.crecv[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine RECV twice", rank);
+  if (w.split_in_dtype != in_dtype)
+    return fail(PPLX_A2A_UNSUPPORTED, "combine RECV must use the expert_y dtype of the SEND phase");
+  LAUNCH_TRY(launch_split_combine_recv(w.dev, w.split, row, rank, in_dtype, out_dtype, stream));
+  w.crecv[rank] = 1;
+  if (++w.n_crecv == R) {
+    std::fill(w.csend.begin(), w.csend.end(), 0);
+    std::fill(w.crecv.begin(), w.crecv.end(), 0);
+    w.n_csend = w.n_crecv = 0;
+  }
+  return PPLX_A2A_OK;
+}
+
 void reset_dispatch_arrivals(pplx_a2a_world &w) {
   std::fill(w.arrived_dispatch.begin(), w.arrived_dispatch.end(), 0);
   w.n_arrived_dispatch = 0;
@@ -406,6 +574,7 @@ int pplx_a2a_world_destroy(pplx_a2a_world_t *w) {
   (void)hipFree(w->dev.tile_cnt);
   (void)hipFree(w->dev.slot_map);
   (void)hipFree(w->dev.faults);
+  free_split(*w);
   delete w;
   return PPLX_A2A_OK;
 }
@@ -444,12 +613,13 @@ int pplx_a2a_dispatch(pplx_a2a_t *h, const pplx_a2a_dispatch_args_t *args, int s
   if (split_mode != PPLX_A2A_SPLIT_NONE && split_mode != PPLX_A2A_SPLIT_SEND &&
       split_mode != PPLX_A2A_SPLIT_RECV)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
-  if (split_mode != PPLX_A2A_SPLIT_NONE)
-    return fail(PPLX_A2A_UNSUPPORTED, "split send/recv dispatch is not available in this build");
   DispatchRank row;
   int st = convert_dispatch(w, h->rank, *args, &row);
   if (st) return st;
   std::lock_guard<std::mutex> lock(w.mu);
+  if (split_mode != PPLX_A2A_SPLIT_NONE) return split_dispatch(w, h->rank, row, split_mode, stream);
+  if (w.n_dsend != 0 || w.n_drecv != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a split dispatch step is still in flight");
   if (w.arrived_dispatch[h->rank])
     return fail(PPLX_A2A_INVALID_STATE,
                 "rank %u called dispatch twice before the other ranks of the step", h->rank);
@@ -467,12 +637,14 @@ int pplx_a2a_combine(pplx_a2a_t *h, const pplx_a2a_combine_args_t *args, int spl
   if (split_mode != PPLX_A2A_SPLIT_NONE && split_mode != PPLX_A2A_SPLIT_SEND &&
       split_mode != PPLX_A2A_SPLIT_RECV)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
-  if (split_mode != PPLX_A2A_SPLIT_NONE)
-    return fail(PPLX_A2A_UNSUPPORTED, "split send/recv combine is not available in this build");
   CombineRank row;
   int st = convert_combine(w, h->rank, *args, &row);
   if (st) return st;
   std::lock_guard<std::mutex> lock(w.mu);
+  if (split_mode != PPLX_A2A_SPLIT_NONE)
+    return split_combine(w, h->rank, row, args->in_dtype, args->out_dtype, split_mode, stream);
+  if (w.n_csend != 0 || w.n_crecv != 0)
+    return fail(PPLX_A2A_INVALID_STATE, "a split combine step is still in flight");
   if (w.arrived_combine[h->rank])
     return fail(PPLX_A2A_INVALID_STATE,
                 "rank %u called combine twice before the other ranks of the step", h->rank);
@@ -495,7 +667,7 @@ int pplx_a2a_world_dispatch(pplx_a2a_world_t *w, const pplx_a2a_dispatch_args_t 
                             void *stream) {
   if (!w || !per_rank) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / per_rank is NULL");
   std::lock_guard<std::mutex> lock(w->mu);
-  if (w->n_arrived_dispatch != 0)
+  if (w->n_arrived_dispatch != 0 || w->n_dsend != 0 || w->n_drecv != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a per-rank dispatch step is still being assembled");
   for (uint32_t r = 0; r < w->dev.R; ++r) {
     int st = convert_dispatch(*w, r, per_rank[r], &w->pend_dispatch[r]);
@@ -508,7 +680,7 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *w, const pplx_a2a_combine_args_t *p
                            void *stream) {
   if (!w || !per_rank) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / per_rank is NULL");
   std::lock_guard<std::mutex> lock(w->mu);
-  if (w->n_arrived_combine != 0)
+  if (w->n_arrived_combine != 0 || w->n_csend != 0 || w->n_crecv != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a per-rank combine step is still being assembled");
   for (uint32_t r = 0; r < w->dev.R; ++r) {
     if (per_rank[r].in_dtype != per_rank[0].in_dtype || per_rank[r].out_dtype != per_rank[0].out_dtype)

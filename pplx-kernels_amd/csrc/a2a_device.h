@@ -77,6 +77,40 @@ struct WorldDev {
   uint32_t *faults;      // [1] sticky fault bits
 };
 
+// Which virtual tokens a routing launch covers and where its results go.
+struct RouteSpan {
+  uint32_t v_begin;       // first virtual token (tiles are counted from here)
+  uint32_t v_count;       // virtual tokens covered
+  uint32_t *tile_cnt;     // [tiles][E]
+  uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
+  // split mode only (one DP group per launch):
+  uint32_t *expert_out;   // [G * M][K] expert of every pair
+  uint32_t *counts_out;   // [E] rows per expert sent by the group
+  uint32_t *offsets_out;  // [E] exclusive prefix of counts_out over experts
+  uint32_t *ntok_out;     // [1] tokens the group sent
+};
+
+// Device state of split send / recv mode: a two-hop path through staging that the world
+// owns.  dispatch SEND packs a group's rows, sorted by expert, into stage_x in the
+// reference's wire format  row | fp32 scales | u32 source token, padded to 16 bytes
+// (csrc/all_to_all/intranode.cpp:41-47, csrc/all_to_all/intranode_dispatch.cu:60-61,148-150);
+// dispatch RECV unpacks into the caller's expert-major outputs.  combine SEND copies expert
+// rows into stage_y, one row per (token, pick); combine RECV reduces them.
+struct SplitDev {
+  uint8_t *stage_x;        // [G][M * K rows][token_stride]
+  uint32_t token_stride;   // round_up(Hb + 4 S + 4, 16)
+  uint32_t tiles_per_group;
+  uint32_t *gtile_cnt;     // [G][tiles_per_group][E]
+  uint32_t *gslot;         // [G * M][K] row of a pair inside its (group, expert) run
+  uint32_t *gexp;          // [G * M][K] expert of a pair
+  uint32_t *gcnt;          // [G][E] rows group g sent to expert e
+  uint32_t *goff;          // [G][E] start of that run inside the group's staging area
+  uint32_t *gbase;         // [G][E] rows of expert e that come from groups before g
+  uint32_t *gntok;         // [G] tokens group g sent
+  uint8_t *stage_y;        // [G * M * K][y_row_bytes]
+  uint64_t y_row_bytes;
+};
+
 // Worlds of up to kInlineRanks ranks pass their rank tables to the kernels as
 // kernel arguments; larger worlds go through the HBM tables (drank / crank),
 // written by bind kernels that take up to kBindBatch rows as arguments each.
@@ -104,6 +138,15 @@ int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stre
 int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *stream);
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
+// Split mode phases of one rank (`row` holds that rank's arguments of the call).
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
+                               uint32_t rank, void *stream);
+int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
+                               uint32_t rank, bool first_of_step, void *stream);
+int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
+                              uint32_t rank, int in_dtype, void *stream);
+int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
+                              uint32_t rank, int in_dtype, int out_dtype, void *stream);
 // True when dispatch runs as the single fused launch for this geometry.
 bool dispatch_is_fused(const WorldDev &w);
 // LDS bytes the routing kernels need for a given geometry.

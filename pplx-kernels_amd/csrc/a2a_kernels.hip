@@ -46,10 +46,12 @@ struct HbmDispatch {
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
 struct InlineCombine {
+  static constexpr bool kStaged = false;
   CombineRank rows[kInlineRanks];
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
 struct HbmCombine {
+  static constexpr bool kStaged = false;
   const CombineRank *rows;
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
@@ -106,6 +108,18 @@ template <> struct SettleAll<16> {
   }
 };
 
+// Split mode: a launch sees only the calling rank's arguments (its peers may not
+// have called yet), whatever rank index is asked for.
+struct SingleDispatch {
+  DispatchRank row;
+  __device__ __forceinline__ const DispatchRank &at(uint32_t) const { return row; }
+};
+struct SingleCombine {
+  static constexpr bool kStaged = true;  // rows come from the world's stage_y, not expert_y
+  CombineRank row;
+  __device__ __forceinline__ const CombineRank &at(uint32_t) const { return row; }
+};
+
 __device__ __forceinline__ uint32_t lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
@@ -150,16 +164,21 @@ __global__ __launch_bounds__(256) void bind_rows(Row *table, Batch b) {
 // the order in which the reference test appends to expert_token_from.  A tile
 // is tile_chunks consecutive chunks of 64 virtual tokens.
 // ---------------------------------------------------------------------------
+// SPLIT = false: one launch routes every DP group and writes out_expert_num_tokens of the
+// owning ranks.  SPLIT = true: the launch routes the span of one DP group from the calling
+// rank's indices alone and leaves group-local results (slot inside (group, expert), expert of
+// each pair, rows per expert and their exclusive prefix over experts) for the later phases.
 template <class DT>
-__global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab) {
+__global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpan span) {
   extern __shared__ uint32_t lds_hist[];
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_hist[e] = 0;
   __syncthreads();
 
-  const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t v = span.v_begin + i;
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  if (g < w.G && t < dispatch_group_tokens(w, tab, g)) {
+  if (i < span.v_count && g < w.G && t < dispatch_group_tokens(w, tab, g)) {
     const uint32_t *idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
@@ -167,12 +186,12 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab) {
     }
   }
   __syncthreads();
-  uint32_t *out = w.tile_cnt + (size_t)blockIdx.x * w.E;
+  uint32_t *out = span.tile_cnt + (size_t)blockIdx.x * w.E;
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) out[e] = lds_hist[e];
 }
 
-template <class DT>
-__global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab) {
+template <class DT, bool SPLIT>
+__global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpan span) {
   // LDS: mask[chunks][E] (one bit per token of the chunk routed to e),
   //      then base[chunks][E] (rows of e taken before the chunk starts).
   extern __shared__ unsigned long long lds_mask[];
@@ -184,10 +203,13 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab) {
 
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t chunk = threadIdx.x / kWave;
-  const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t v = span.v_begin + i;
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  const bool live = g < w.G && t < dispatch_group_tokens(w, tab, g);
+  const bool in_span = i < span.v_count && g < w.G;
+  const uint32_t n_group = in_span ? dispatch_group_tokens(w, tab, g) : 0;
+  const bool live = in_span && t < n_group;
   const uint32_t *idx = nullptr;
   bool bad_expert = false;
   if (live) {
@@ -204,25 +226,30 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab) {
   __syncthreads();
 
   // Per expert: rows taken by earlier tiles, then running prefix over chunks.
+  const bool last_tile = blockIdx.x == gridDim.x - 1;
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
     uint32_t running = 0;
-    for (uint32_t tile = 0; tile < blockIdx.x; ++tile) running += w.tile_cnt[(size_t)tile * w.E + e];
+    for (uint32_t tile = 0; tile < blockIdx.x; ++tile) running += span.tile_cnt[(size_t)tile * w.E + e];
     for (uint32_t c = 0; c < chunks; ++c) {
       lds_base[c * w.E + e] = running;
       running += __popcll(lds_mask[(size_t)c * w.E + e]);
     }
-    if (blockIdx.x == gridDim.x - 1) {
-      // out_expert_num_tokens of the owning rank
-      // (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).
-      const DispatchRank &owner = tab.at(e / w.L);
-      owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
+    if (last_tile) {
+      if (SPLIT) {
+        span.counts_out[e] = running;
+      } else {
+        // out_expert_num_tokens of the owning rank
+        // (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).
+        const DispatchRank &owner = tab.at(e / w.L);
+        owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
+      }
     }
   }
   __syncthreads();
 
   if (live) {
     const unsigned long long below = (1ull << lane) - 1ull;
-    uint32_t *out = w.slot_map + (size_t)v * w.K;
+    uint32_t *out = span.slot_out + (size_t)v * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
       uint32_t slot = kInvalidSlot;
@@ -230,8 +257,34 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab) {
         slot = lds_base[chunk * w.E + e] + __popcll(lds_mask[(size_t)chunk * w.E + e] & below);
       }
       out[k] = slot;
+      if (SPLIT) span.expert_out[(size_t)v * w.K + k] = e;
     }
     if (bad_expert) atomicOr(w.faults, kFaultBadExpert);
+  }
+
+  if (SPLIT && last_tile) {
+    // Exclusive prefix of counts_out over experts: where each expert's rows start in the
+    // group's compact staging area.  counts_out was written by this workgroup above.
+    __syncthreads();
+    uint32_t *scan = reinterpret_cast<uint32_t *>(lds_mask);  // blockDim entries, LDS is free now
+    const uint32_t per_thread = (w.E + blockDim.x - 1) / blockDim.x;
+    const uint32_t e0 = threadIdx.x * per_thread;
+    uint32_t local = 0;
+    for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) local += span.counts_out[e];
+    scan[threadIdx.x] = local;
+    __syncthreads();
+    for (uint32_t step = 1; step < blockDim.x; step *= 2) {
+      const uint32_t add = threadIdx.x >= step ? scan[threadIdx.x - step] : 0;
+      __syncthreads();
+      scan[threadIdx.x] += add;
+      __syncthreads();
+    }
+    uint32_t running = scan[threadIdx.x] - local;
+    for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) {
+      span.offsets_out[e] = running;
+      running += span.counts_out[e];
+    }
+    if (threadIdx.x == 0) *span.ntok_out = dispatch_group_tokens(w, tab, span.v_begin / w.M);
   }
 }
 
@@ -549,15 +602,18 @@ __device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, f
 // eight loads; with KK in {1, 2, 4} the wave takes VPL = 8 / KK vectors per lane so
 // that eight row loads per lane are in flight for small top-k too.
 template <typename T, typename U, class CT, int KK, int VPL>
-__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments) {
+__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments,
+                                                      uint32_t first_rank, uint32_t rank_count,
+                                                      const uint8_t *stage_y, uint64_t stage_row_bytes) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
                                                        threadIdx.x / kWave);
   const uint32_t token = wave / segments;
   const uint32_t segment = wave - token * segments;
-  const uint32_t r = token / w.M;
-  const uint32_t t = token - r * w.M;
-  if (r >= w.R) return;
+  const uint32_t r_local = token / w.M;
+  const uint32_t t = token - r_local * w.M;
+  if (r_local >= rank_count) return;
+  const uint32_t r = first_rank + r_local;
   const CombineRank &c = tab.at(r);
   if (t >= combine_rank_tokens(w, c)) return;
 
@@ -568,7 +624,13 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
     const uint32_t e = c.indices[(size_t)t * w.K + lane];
     const uint32_t slot = w.slot_map[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
     weight = c.weights[(int64_t)t * c.w_stride_row + lane];
-    if (e < w.E && slot != kInvalidSlot) {
+    if (CT::kStaged) {
+      // combine SEND left the row of (token, pick) in the staging area.
+      if (e < w.E && slot != kInvalidSlot) {
+        row = reinterpret_cast<uint64_t>(stage_y) +
+              (((uint64_t)(r / w.dp) * w.M + t) * w.K + lane) * stage_row_bytes;
+      }
+    } else if (e < w.E && slot != kInvalidSlot) {
       const CombineRank &owner = tab.at(e / w.L);
       if (slot < owner.y_rows) {
         row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
@@ -634,6 +696,212 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
 }
 
 // ---------------------------------------------------------------------------
+// Split send / recv mode (two hops through world-owned staging).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint8_t *stage_row(const WorldDev &w, const SplitDev &sp, uint32_t g,
+                                              uint32_t position) {
+  return sp.stage_x + ((uint64_t)g * w.M * w.K + position) * sp.token_stride;
+}
+
+// dispatch SEND, second half: one wave per token of the calling rank's share packs
+// row | scales | source token into the group's staging area, grouped by expert.
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g, uint32_t member,
+                                                  SplitDev sp) {
+  const uint32_t lane = lane_id();
+  const uint32_t t = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
+  if (t >= w.M || t % w.dp != member || t >= sp.gntok[g]) return;
+  const DispatchRank &src = tab.at(0);
+  const uint32_t nvec = w.Hb / 16;
+  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
+  u32x4 x[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    uint32_t j = lane + i * kWave;
+    if (!EXACT) j = j < nvec ? j : nvec - 1;
+    x[i] = row[j];
+  }
+  const uint32_t S = w.S;
+  const float *srow = S ? src.dp_xs + (int64_t)t * src.dp_xs_stride_row : nullptr;
+  uint64_t dst = 0;
+  if (lane < w.K) {
+    const size_t pair = ((size_t)g * w.M + t) * w.K + lane;
+    const uint32_t e = sp.gexp[pair];
+    if (e < w.E) dst = reinterpret_cast<uint64_t>(stage_row(w, sp, g, sp.goff[(size_t)g * w.E + e] + sp.gslot[pair]));
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) settle(x[i]);
+  settle(dst);
+  for (uint32_t k = 0; k < w.K; ++k) {
+    const uint64_t p = read_lane64(dst, k);
+    if (p == 0) continue;
+    PPLX_GLOBAL u32x4 *out = global_ptr<u32x4>(p);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const uint32_t j = lane + i * kWave;
+      if (EXACT || j < nvec) out[j] = x[i];
+    }
+    PPLX_GLOBAL float *sout = global_ptr<float>(p + w.Hb);
+    for (uint32_t j = lane; j < S; j += kWave) sout[j] = srow[(int64_t)j * src.dp_xs_stride_elem];
+    if (lane == 0) *global_ptr<uint32_t>(p + w.Hb + 4ull * S) = t;
+  }
+}
+
+// First dispatch RECV of a step: rows of every expert that come from earlier groups.
+__global__ __launch_bounds__(256) void split_bases(WorldDev w, SplitDev sp) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= w.E) return;
+  uint32_t running = 0;
+  for (uint32_t g = 0; g < w.G; ++g) {
+    sp.gbase[(size_t)g * w.E + e] = running;
+    running += sp.gcnt[(size_t)g * w.E + e];
+  }
+}
+
+// ... and the slot map that combine reads: slot = rows from earlier groups + slot in the group.
+__global__ __launch_bounds__(256) void split_finalize(WorldDev w, SplitDev sp) {
+  const uint64_t pair = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (pair >= (uint64_t)w.G * w.M * w.K) return;
+  const uint32_t v = (uint32_t)(pair / w.K);
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (t >= sp.gntok[g]) return;
+  const uint32_t e = sp.gexp[pair];
+  w.slot_map[pair] = e < w.E ? sp.gbase[(size_t)g * w.E + e] + sp.gslot[pair] : kInvalidSlot;
+}
+
+// dispatch RECV of rank d: workgroup (local expert, group) copies that run of staged rows
+// into out_expert_x / out_expert_x_scale; blockIdx.y spreads long runs.
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t d, SplitDev sp) {
+  const uint32_t lane = lane_id();
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t el = blockIdx.x / w.G;
+  const uint32_t g = blockIdx.x - el * w.G;
+  const uint32_t e = d * w.L + el;
+  const DispatchRank &dst = tab.at(0);
+  const size_t ge = (size_t)g * w.E + e;
+  const uint32_t count = sp.gcnt[ge], offset = sp.goff[ge], base = sp.gbase[ge];
+  if (g == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    const size_t last = (size_t)(w.G - 1) * w.E + e;
+    dst.out_num_tokens[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)(sp.gbase[last] + sp.gcnt[last]);
+  }
+  const uint32_t nvec = w.Hb / 16;
+  const uint32_t S = w.S;
+  for (uint32_t i = blockIdx.y * (blockDim.x / kWave) + wave; i < count; i += gridDim.y * (blockDim.x / kWave)) {
+    const uint32_t slot = base + i;
+    if (slot >= dst.x_rows) {
+      if (lane == 0) atomicOr(w.faults, kFaultRowDropped);
+      continue;
+    }
+    const uint8_t *src = stage_row(w, sp, g, offset + i);
+    const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
+    u32x4 *out = reinterpret_cast<u32x4 *>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
+                                           (int64_t)slot * dst.x_stride_row);
+    u32x4 x[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      uint32_t j = lane + v * kWave;
+      if (!EXACT) j = j < nvec ? j : nvec - 1;
+      x[v] = row[j];
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const uint32_t j = lane + v * kWave;
+      if (EXACT || j < nvec) __builtin_nontemporal_store(x[v], out + j);
+    }
+    if (S) {
+      const float *sin = reinterpret_cast<const float *>(src + w.Hb);
+      float *sout = dst.expert_xs + (int64_t)el * dst.xs_stride_expert + (int64_t)slot * dst.xs_stride_row;
+      for (uint32_t j = lane; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
+    }
+  }
+}
+
+// Rows beyond the register variants: plain streaming loops, one workgroup per staged row.
+template <class DT>
+__global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, uint32_t g, uint32_t member,
+                                                       SplitDev sp) {
+  const uint32_t t = blockIdx.x;
+  if (t >= w.M || t % w.dp != member || t >= sp.gntok[g]) return;
+  const DispatchRank &src = tab.at(0);
+  const uint32_t nvec = w.Hb / 16;
+  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
+  for (uint32_t k = 0; k < w.K; ++k) {
+    const size_t pair = ((size_t)g * w.M + t) * w.K + k;
+    const uint32_t e = sp.gexp[pair];
+    if (e >= w.E) continue;
+    uint8_t *p = stage_row(w, sp, g, sp.goff[(size_t)g * w.E + e] + sp.gslot[pair]);
+    u32x4 *out = reinterpret_cast<u32x4 *>(p);
+    for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
+    float *sout = reinterpret_cast<float *>(p + w.Hb);
+    for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) {
+      sout[j] = src.dp_xs[(int64_t)t * src.dp_xs_stride_row + (int64_t)j * src.dp_xs_stride_elem];
+    }
+    if (threadIdx.x == 0) *reinterpret_cast<uint32_t *>(p + w.Hb + 4ull * w.S) = t;
+  }
+}
+
+template <class DT>
+__global__ __launch_bounds__(256) void split_unpack_long(WorldDev w, DT tab, uint32_t d, SplitDev sp) {
+  const uint32_t el = blockIdx.x / w.G;
+  const uint32_t g = blockIdx.x - el * w.G;
+  const uint32_t e = d * w.L + el;
+  const DispatchRank &dst = tab.at(0);
+  const size_t ge = (size_t)g * w.E + e;
+  const uint32_t count = sp.gcnt[ge], offset = sp.goff[ge], base = sp.gbase[ge];
+  if (g == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    const size_t last = (size_t)(w.G - 1) * w.E + e;
+    dst.out_num_tokens[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)(sp.gbase[last] + sp.gcnt[last]);
+  }
+  const uint32_t nvec = w.Hb / 16;
+  for (uint32_t i = blockIdx.y; i < count; i += gridDim.y) {
+    const uint32_t slot = base + i;
+    if (slot >= dst.x_rows) {
+      if (threadIdx.x == 0) atomicOr(w.faults, kFaultRowDropped);
+      continue;
+    }
+    const uint8_t *src = stage_row(w, sp, g, offset + i);
+    const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
+    u32x4 *out = reinterpret_cast<u32x4 *>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
+                                           (int64_t)slot * dst.x_stride_row);
+    for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
+    const float *sin = reinterpret_cast<const float *>(src + w.Hb);
+    float *sout = dst.expert_xs + (int64_t)el * dst.xs_stride_expert + (int64_t)slot * dst.xs_stride_row;
+    for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
+  }
+}
+
+// combine SEND of rank d: one wave per (token, pick) whose expert d owns copies that
+// expert_y row into the pair's staging row (the reference copies it into the source
+// rank's inbox, csrc/all_to_all/intranode_combine.cu:77-111).
+template <class CT>
+__global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, uint32_t d, SplitDev sp,
+                                                          uint32_t elem_bytes) {
+  const uint32_t lane = lane_id();
+  const uint64_t pair = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
+  if (pair >= (uint64_t)w.G * w.M * w.K) return;
+  const uint32_t v = (uint32_t)(pair / w.K);
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (t >= sp.gntok[g]) return;
+  const uint32_t e = sp.gexp[pair];
+  if (e >= w.E || e / w.L != d) return;
+  const uint32_t slot = w.slot_map[pair];
+  const CombineRank &own = tab.at(0);
+  if (slot >= own.y_rows) {
+    if (lane == 0) atomicOr(w.faults, kFaultBadSlot);
+    return;
+  }
+  const uint8_t *src = reinterpret_cast<const uint8_t *>(own.expert_y) +
+                       ((int64_t)(e % w.L) * own.y_stride_expert + (int64_t)slot * own.y_stride_row) * elem_bytes;
+  const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
+  u32x4 *out = reinterpret_cast<u32x4 *>(sp.stage_y + pair * sp.y_row_bytes);
+  const uint32_t nvec = (uint32_t)(sp.y_row_bytes / 16);
+  for (uint32_t j = lane; j < nvec; j += kWave) out[j] = __builtin_nontemporal_load(row + j);
+}
+
+// ---------------------------------------------------------------------------
 // Launch helpers
 // ---------------------------------------------------------------------------
 InlineDispatch make_inline(const WorldDev &w, const DispatchRank *rows) {
@@ -648,23 +916,24 @@ InlineCombine make_inline(const WorldDev &w, const CombineRank *rows) {
   return t;
 }
 
-template <class DT>
-int launch_route_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+template <class DT, bool SPLIT>
+int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
   const uint32_t block = w.tile_chunks * kWave;
-  if (w.num_tiles > 1) {
-    hipLaunchKernelGGL(route_count<DT>, dim3(w.num_tiles), dim3(block), w.E * sizeof(uint32_t), s, w, tab);
+  const uint32_t tiles = (span.v_count + block - 1) / block;
+  if (tiles > 1) {
+    hipLaunchKernelGGL(route_count<DT>, dim3(tiles), dim3(block), w.E * sizeof(uint32_t), s, w, tab, span);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return (int)err;
   }
-  hipLaunchKernelGGL(route_slots<DT>, dim3(w.num_tiles), dim3(block), route_lds_bytes(w.E, w.tile_chunks),
-                     s, w, tab);
+  hipLaunchKernelGGL((route_slots<DT, SPLIT>), dim3(tiles), dim3(block),
+                     route_lds_bytes(w.E, w.tile_chunks), s, w, tab, span);
   return (int)hipGetLastError();
 }
 
 // Picks the register variant for the row size and launches KERNEL<NV, EXACT, DT>.
 // Rows beyond 8 KiB exist only for dispatch_scatter (PPLX_LAUNCH_LARGE_ROW_VARIANT).
 #define PPLX_LAUNCH_ROW_VARIANT(KERNEL, NV, EXACT)                                               \
-  hipLaunchKernelGGL((KERNEL<NV, EXACT, DT>), grid, block, lds, s, w, tab, ksplit, kper)
+  hipLaunchKernelGGL((KERNEL<NV, EXACT, DT>), grid, block, lds, s, w, tab, PPLX_ROW_KERNEL_ARGS)
 
 #define PPLX_DISPATCH_ROW_VARIANTS(KERNEL)                                                       \
   do {                                                                                           \
@@ -707,6 +976,7 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint64_t waves = (uint64_t)tokens * ksplit;
   const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
   const uint32_t lds = 0;
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL)                                                    \
   do {                                                                                           \
     if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                              \
@@ -714,6 +984,7 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   } while (0)
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
+#undef PPLX_ROW_KERNEL_ARGS
   return (int)hipGetLastError();
 }
 
@@ -726,46 +997,56 @@ int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint32_t tokens_per_block = kWaves / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
   const uint32_t lds = (w.E + w.G + tokens_per_block * w.K) * sizeof(uint32_t);
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
+#undef PPLX_ROW_KERNEL_ARGS
   return (int)hipGetLastError();
 }
 
 template <class DT>
 int launch_dispatch_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   if (dispatch_is_fused(w)) return launch_fused_t(w, tab, s);
-  int err = launch_route_t(w, tab, s);
+  RouteSpan span{};
+  span.v_begin = 0;
+  span.v_count = w.G * w.M;
+  span.tile_cnt = w.tile_cnt;
+  span.slot_out = w.slot_map;
+  int err = launch_route_t<DT, false>(w, tab, span, s);
   if (err) return err;
   return launch_scatter_t(w, tab, s);
 }
 
 template <typename T, typename U, class CT>
-int launch_combine_k(const WorldDev &w, const CT &tab, hipStream_t s) {
+int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
+                     const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
   const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
   const uint32_t vpl = w.K == 1 ? 8 : w.K == 2 ? 4 : w.K == 4 ? 2 : 1;
   const uint32_t segments = (nvec_segments + vpl - 1) / vpl;
-  const uint64_t waves = (uint64_t)w.R * w.M * segments;
+  const uint64_t waves = (uint64_t)rank_count * w.M * segments;
   const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
   switch (w.K) {
-    case 1: hipLaunchKernelGGL((combine_gather<T, U, CT, 1, 8>), grid, block, 0, s, w, tab, segments); break;
-    case 2: hipLaunchKernelGGL((combine_gather<T, U, CT, 2, 4>), grid, block, 0, s, w, tab, segments); break;
-    case 4: hipLaunchKernelGGL((combine_gather<T, U, CT, 4, 2>), grid, block, 0, s, w, tab, segments); break;
-    default: hipLaunchKernelGGL((combine_gather<T, U, CT, 0, 1>), grid, block, 0, s, w, tab, segments); break;
+    case 1: hipLaunchKernelGGL((combine_gather<T, U, CT, 1, 8>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    case 2: hipLaunchKernelGGL((combine_gather<T, U, CT, 2, 4>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    case 4: hipLaunchKernelGGL((combine_gather<T, U, CT, 4, 2>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    default: hipLaunchKernelGGL((combine_gather<T, U, CT, 0, 1>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
   }
   return (int)hipGetLastError();
 }
 
 template <class CT>
-int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s) {
+int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s,
+                     uint32_t first_rank, uint32_t rank_count, const uint8_t *stage_y = nullptr,
+                     uint64_t stage_row_bytes = 0) {
   // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
   switch (in_dtype * 4 + out_dtype) {
-    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, s);
-    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, s);
-    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, s);
-    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, s);
-    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, s);
-    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, s);
+    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
     default: return (int)hipErrorInvalidValue;
   }
 }
@@ -776,7 +1057,9 @@ int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dty
 // Launchers
 // ---------------------------------------------------------------------------
 uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
-  return tile_chunks * num_experts * (uint32_t)(sizeof(unsigned long long) + sizeof(uint32_t));
+  const uint32_t tables = tile_chunks * num_experts * (uint32_t)(sizeof(unsigned long long) + sizeof(uint32_t));
+  const uint32_t scan = tile_chunks * kWave * (uint32_t)sizeof(uint32_t);  // split mode's block scan
+  return tables > scan ? tables : scan;
 }
 
 bool dispatch_is_fused(const WorldDev &w) {
@@ -804,11 +1087,86 @@ int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *st
   return launch_dispatch_t(w, HbmDispatch{w.drank}, (hipStream_t)stream);
 }
 
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
+                               uint32_t rank, void *stream) {
+  typedef SingleDispatch DT;
+  hipStream_t s = (hipStream_t)stream;
+  const DT tab{row};
+  const uint32_t g = rank / w.dp, member = rank % w.dp;
+  RouteSpan span{};
+  span.v_begin = g * w.M;
+  span.v_count = w.M;
+  span.tile_cnt = sp.gtile_cnt + (size_t)g * sp.tiles_per_group * w.E;
+  span.slot_out = sp.gslot;
+  span.expert_out = sp.gexp;
+  span.counts_out = sp.gcnt + (size_t)g * w.E;
+  span.offsets_out = sp.goff + (size_t)g * w.E;
+  span.ntok_out = sp.gntok + g;
+  int err = launch_route_t<DT, true>(w, tab, span, s);
+  if (err) return err;
+  const uint32_t lds = 0;
+  if ((w.Hb / 16 + kWave - 1) / kWave > 8) {
+    hipLaunchKernelGGL(split_pack_long<DT>, dim3(w.M), dim3(256), 0, s, w, tab, g, member, sp);
+    return (int)hipGetLastError();
+  }
+  const dim3 grid((w.M + 3) / 4), block(256);
+#define PPLX_ROW_KERNEL_ARGS g, member, sp
+#define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
+  PPLX_DISPATCH_ROW_VARIANTS(split_pack);
+#undef PPLX_LAUNCH_LARGE_ROW_VARIANT
+#undef PPLX_ROW_KERNEL_ARGS
+  return (int)hipGetLastError();
+}
+
+int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
+                               uint32_t rank, bool first_of_step, void *stream) {
+  typedef SingleDispatch DT;
+  hipStream_t s = (hipStream_t)stream;
+  const DT tab{row};
+  if (first_of_step) {
+    hipLaunchKernelGGL(split_bases, dim3((w.E + 255) / 256), dim3(256), 0, s, w, sp);
+    const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
+    hipLaunchKernelGGL(split_finalize, dim3((uint32_t)((pairs + 255) / 256)), dim3(256), 0, s, w, sp);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return (int)err;
+  }
+  const uint32_t lds = 0;
+  // enough row groups that a hot expert's run is shared by many workgroups
+  const uint32_t spread = w.M >= 2048 ? 16 : w.M >= 256 ? 4 : 1;
+  const dim3 grid(w.L * w.G, spread), block(256);
+  if ((w.Hb / 16 + kWave - 1) / kWave > 8) {
+    hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, rank, sp);
+    return (int)hipGetLastError();
+  }
+#define PPLX_ROW_KERNEL_ARGS rank, sp
+#define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
+  PPLX_DISPATCH_ROW_VARIANTS(split_unpack);
+#undef PPLX_LAUNCH_LARGE_ROW_VARIANT
+#undef PPLX_ROW_KERNEL_ARGS
+  return (int)hipGetLastError();
+}
+
+int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
+                              uint32_t rank, int in_dtype, void *stream) {
+  const SingleCombine tab{row};
+  const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
+  const uint32_t elem_bytes = in_dtype == 0 ? 4u : 2u;
+  hipLaunchKernelGGL(split_combine_send<SingleCombine>, dim3((uint32_t)((pairs + 3) / 4)), dim3(256), 0,
+                     (hipStream_t)stream, w, tab, rank, sp, elem_bytes);
+  return (int)hipGetLastError();
+}
+
+int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
+                              uint32_t rank, int in_dtype, int out_dtype, void *stream) {
+  return launch_combine_t(w, SingleCombine{row}, in_dtype, out_dtype, (hipStream_t)stream, rank, 1,
+                          sp.stage_y, sp.y_row_bytes);
+}
+
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream) {
   if (inline_rows)
-    return launch_combine_t(w, make_inline(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream);
-  return launch_combine_t(w, HbmCombine{w.crank}, in_dtype, out_dtype, (hipStream_t)stream);
+    return launch_combine_t(w, make_inline(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream, 0, w.R);
+  return launch_combine_t(w, HbmCombine{w.crank}, in_dtype, out_dtype, (hipStream_t)stream, 0, w.R);
 }
 
 }  // namespace pplx_amd

@@ -489,10 +489,11 @@ def _dispatch(
     mode = split_mode(do_send, do_recv)
     with torch.cuda.device(indices.device):
         check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    _handle_world[fptr].hold(
-        "dispatch",
-        (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
-    )
+    if mode == SPLIT_NONE:
+        _handle_world[fptr].hold(
+            "dispatch",
+            (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
+        )
 
 
 def _combine(
@@ -510,7 +511,8 @@ def _combine(
     mode = split_mode(do_send, do_recv)
     with torch.cuda.device(indices.device):
         check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    _handle_world[fptr].hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
+    if mode == SPLIT_NONE:
+        _handle_world[fptr].hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
 
 
 def _fake_dispatch(*args, **kwargs) -> None:

@@ -454,6 +454,117 @@ def test_out_of_range_expert_is_ignored_and_reported():
 
 
 # ---------------------------------------------------------------------------
+# Split send / recv (do_send / do_recv), the sequence of the reference's C++ bench
+# (csrc/all_to_all/bench_all_to_all.cpp:183-203)
+# ---------------------------------------------------------------------------
+def _make_ranks(spec, name):
+    from pplx_kernels import AllToAll
+
+    return [
+        AllToAll.intranode(
+            spec.max_num_tokens, spec.num_experts, spec.experts_per_token, r, spec.world_size, spec.dp_size,
+            spec.hidden_dim, spec.hidden_dim_bytes, spec.hidden_dim_scale_bytes, group_name=name,
+        )  # fmt: skip
+        for r in range(spec.world_size)
+    ]
+
+
+def _dispatch_kw(step, r):
+    return dict(
+        out_expert_num_tokens=step.expert_num_tokens[r], out_expert_x=step.expert_x[r],
+        out_expert_x_scale=step.expert_x_scale[r], dp_x=step.dp_x[r], dp_x_scale=step.dp_x_scale[r],
+        indices=step.indices[r], bound_m=step.bound_m[r],
+    )  # fmt: skip
+
+
+def _combine_kw(step, r):
+    return dict(
+        out_tokens=step.out_tokens[r], indices=step.indices[r], weights=step.weights[r],
+        expert_y=step.expert_y[r], bound_m=step.bound_m[r],
+    )  # fmt: skip
+
+
+@pytest.mark.parametrize(
+    "kw",
+    [
+        dict(name="split-bf16"),
+        dict(name="split-fp8", in_dtype=FP8, hidden_dim=1024),
+        dict(name="split-dp2", dp_size=2, in_dtype=FP8, hidden_dim=512),
+        dict(name="split-tiles", max_num_tokens=1300, world_size=2, num_experts=8, hidden_dim=64),
+        dict(name="split-longrow", hidden_dim=20480, max_num_tokens=6),
+        dict(name="split-f32y", expert_y_dtype=torch.float32, out_dtype=torch.float16),
+    ],
+    ids=lambda kw: kw["name"],
+)
+def test_split_send_recv(kw):
+    spec = _small_spec(**kw)
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    ranks = _make_ranks(spec, kw["name"])
+    R = spec.world_size
+    for round_ in range(2):  # twice: the per-step state must reset itself
+        step.expert_x_all.view(torch.uint8).fill_(0)
+        step.expert_num_tokens_all.fill_(-1)
+        saved = [x.clone() for x in step.dp_x]
+        for r in range(R):
+            ranks[r].dispatch(**_dispatch_kw(step, r), do_send=True, do_recv=False)
+        # SEND has consumed the inputs and must not have touched the outputs yet
+        torch.cuda.synchronize()
+        assert int(step.expert_x_all.view(torch.uint8).max()) == 0
+        assert int(step.expert_num_tokens_all.max()) == -1
+        for x in step.dp_x:
+            x.view(torch.uint8).fill_(0x7F)
+        for r in reversed(range(R)):
+            ranks[r].dispatch(**_dispatch_kw(step, r), do_send=False, do_recv=True)
+        for x, s_ in zip(step.dp_x, saved):
+            x.copy_(s_)
+        expected = check_dispatch_against_oracle(step)
+
+        gen = torch.Generator(device="cuda").manual_seed(round_)
+        step.expert_y_all.copy_(torch.randn(step.expert_y_all.shape, generator=gen, device="cuda"))
+        y_saved = step.expert_y_all.clone()
+        for t in step.out_tokens:
+            t.fill_(float("nan"))
+        for r in range(R):
+            ranks[r].combine(**_combine_kw(step, r), do_send=True, do_recv=False)
+        torch.cuda.synchronize()
+        assert all(torch.isnan(t).all() for t in step.out_tokens)  # nothing delivered before RECV
+        step.expert_y_all.fill_(7.0)  # SEND has consumed expert_y
+        for r in range(R):
+            ranks[r].combine(**_combine_kw(step, r), do_send=False, do_recv=True)
+        torch.cuda.synchronize()
+        step.expert_y_all.copy_(y_saved)
+        check_combine_against_oracle(step, expected.slot_map)
+    for a in ranks:
+        a.destroy()
+
+
+def test_split_order_is_enforced():
+    spec = _small_spec(name="split-order", tokens="max")
+    step = DeviceStep(spec, generate(spec))
+    ranks = _make_ranks(spec, "split-order")
+    ranks[0].dispatch(**_dispatch_kw(step, 0), do_send=True, do_recv=False)
+    with pytest.raises(RuntimeError, match="before every rank's SEND"):
+        ranks[0].dispatch(**_dispatch_kw(step, 0), do_send=False, do_recv=True)
+    with pytest.raises(RuntimeError, match="SEND twice"):
+        ranks[0].dispatch(**_dispatch_kw(step, 0), do_send=True, do_recv=False)
+    with pytest.raises(RuntimeError, match="split dispatch step is still in flight"):
+        ranks[1].dispatch(**_dispatch_kw(step, 1))
+    for r in range(1, spec.world_size):
+        ranks[r].dispatch(**_dispatch_kw(step, r), do_send=True, do_recv=False)
+    for r in range(spec.world_size):
+        ranks[r].dispatch(**_dispatch_kw(step, r), do_send=False, do_recv=True)
+    check_dispatch_against_oracle(step)
+    # after a complete split step the fused mode works again on the same world
+    step.expert_x_all.view(torch.uint8).fill_(0)
+    for r in range(spec.world_size):
+        ranks[r].dispatch(**_dispatch_kw(step, r))
+    check_dispatch_against_oracle(step)
+    for a in ranks:
+        a.destroy()
+
+
+# ---------------------------------------------------------------------------
 # hipGraph replay (decode shape)
 # ---------------------------------------------------------------------------
 def test_graph_replay_decode_shape():
