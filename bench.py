@@ -33,6 +33,10 @@ for _p in (os.path.join(ROOT, "pplx-kernels_amd"), ROOT):
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 LLC_BYTES = 256 << 20
+# HBM bytes per combine_gather launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+# scaled by a copy of known size in the same run (profiles/hbm_traffic_<workload>.txt); counters
+# cannot be read from inside this script, so the figure is carried as a constant per workload.
+MEASURED_COMBINE_TRAFFIC_BYTES = {"C2": 133.0e6, "C5": 4391.9e6}
 
 
 def build_steps(spec, groups, cap, n_sets):
@@ -276,7 +280,7 @@ def main() -> None:
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": comb_b / kernel_us / 1e3 / HBM_PEAK_GBPS,
-        "traffic": None,
+        "traffic": MEASURED_COMBINE_TRAFFIC_BYTES.get(args.workload),
         "bytes_per_launch": comb_b,
         "avg_launch_us": kernel_us,
         "launches_timed": reps * n_sets * launches_per_graph,
