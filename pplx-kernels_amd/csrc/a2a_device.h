@@ -112,10 +112,12 @@ struct SplitDev {
 };
 
 // Worlds of up to kInlineRanks ranks pass their rank tables to the kernels as
-// kernel arguments; larger worlds go through the HBM tables (drank / crank),
-// written by bind kernels that take up to kBindBatch rows as arguments each.
-constexpr uint32_t kInlineRanks = 8;
-constexpr uint32_t kBindBatch = 16;
+// kernel arguments (9 KiB for dispatch, 5 KiB for combine; HIP on gfx950 takes kernel
+// arguments well beyond 4 KiB, eagerly and as graph nodes); larger worlds go through the
+// HBM tables (drank / crank), written by bind kernels that take up to kBindBatch rows as
+// arguments each.
+constexpr uint32_t kInlineRanks = 64;
+constexpr uint32_t kBindBatch = 64;
 // Steps with at most this many (token, pick) pairs dispatch in one fused launch.
 constexpr uint32_t kFusedMaxPairs = 16384;
 

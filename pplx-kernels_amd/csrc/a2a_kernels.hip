@@ -290,36 +290,43 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
 
 // ---------------------------------------------------------------------------
 // Row fan-out shared by dispatch_scatter and dispatch_fused.  The calling wave
-// owns token (g, t); lane k passes the slot of pick k in `slot`.  The row is
-// read once into NV 16-byte registers per lane and stored for picks [k0, k1).
-// EXACT: the row is exactly NV * 64 vectors, so nothing is predicated.
+// owns one token; the row is read once into NV 16-byte registers per lane
+// (load_row) and stored for picks [k0, k1) (store_row), lane k passing the slot of
+// pick k.  EXACT: the row is exactly NV * 64 vectors, so nothing is predicated.
 // ---------------------------------------------------------------------------
-template <int NV, bool EXACT, class DT>
-__device__ __forceinline__ void fan_out_row(const WorldDev &w, const DT &tab, uint32_t g, uint32_t t,
-                                            uint32_t lane, uint32_t slot, uint32_t k0, uint32_t k1,
-                                            bool report) {
-  // The sender of token t inside its DP group (csrc/all_to_all/intranode_dispatch.cu:97).
-  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+template <int NV>
+struct RowRegs {
+  u32x4 x[NV];   // the row, 16 bytes per lane per register
+  float sc;      // scale `lane` of the row (lanes >= S hold a copy of the last one)
+};
+
+// First half: issues the loads of row t of `src`; needs t < src.m only.
+template <int NV, bool EXACT>
+__device__ __forceinline__ void load_row(const WorldDev &w, const DispatchRank &src, uint32_t t,
+                                         uint32_t lane, RowRegs<NV> &regs) {
   const uint32_t nvec = w.Hb / 16;
   const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
-
-  u32x4 x[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     uint32_t j = lane + i * kWave;
     if (!EXACT) j = j < nvec ? j : nvec - 1;  // clamp: loads stay unconditional
-    x[i] = row[j];
+    regs.x[i] = row[j];
   }
-  const uint32_t S = w.S;
-  const float *srow = nullptr;
-  float sc = 0.f;
-  if (S) {
-    srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
-    const uint32_t j = lane < S ? lane : S - 1;
-    sc = srow[(int64_t)j * src.dp_xs_stride_elem];
+  regs.sc = 0.f;
+  if (w.S) {
+    const uint32_t j = lane < w.S ? lane : w.S - 1;
+    regs.sc = src.dp_xs[(int64_t)t * src.dp_xs_stride_row + (int64_t)j * src.dp_xs_stride_elem];
   }
+}
 
-  // Lane k resolves the destination of pick k.
+// Second half: lane k resolves the destination of pick k from `slot`, then the row is stored
+// for picks [k0, k1).
+template <int NV, bool EXACT, class DT>
+__device__ __forceinline__ void store_row(const WorldDev &w, const DT &tab, const DispatchRank &src,
+                                          uint32_t t, uint32_t lane, uint32_t slot, uint32_t k0,
+                                          uint32_t k1, bool report, RowRegs<NV> &regs) {
+  const uint32_t nvec = w.Hb / 16;
+  const uint32_t S = w.S;
   uint64_t dst_row = 0, dst_scale = 0;
   int64_t dst_scale_step = 0;
   if (lane < w.K) {
@@ -342,8 +349,8 @@ __device__ __forceinline__ void fan_out_row(const WorldDev &w, const DT &tab, ui
   }
 
 #pragma unroll
-  for (int i = 0; i < NV; ++i) settle(x[i]);
-  settle(sc);
+  for (int i = 0; i < NV; ++i) settle(regs.x[i]);
+  settle(regs.sc);
   settle(dst_row);
   settle(dst_scale);
   settle(dst_scale_step);
@@ -355,14 +362,17 @@ __device__ __forceinline__ void fan_out_row(const WorldDev &w, const DT &tab, ui
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const uint32_t j = lane + i * kWave;
-      if (EXACT || j < nvec) __builtin_nontemporal_store(x[i], out + j);
+      if (EXACT || j < nvec) __builtin_nontemporal_store(regs.x[i], out + j);
     }
     if (S) {
       PPLX_GLOBAL float *sout = global_ptr<float>(read_lane64(dst_scale, k));
       const int64_t step = (int64_t)read_lane64((uint64_t)dst_scale_step, k);
-      if (lane < S) __builtin_nontemporal_store(sc, sout + (int64_t)lane * step);
-      for (uint32_t j = lane + kWave; j < S; j += kWave) {
-        sout[(int64_t)j * step] = srow[(int64_t)j * src.dp_xs_stride_elem];
+      if (lane < S) __builtin_nontemporal_store(regs.sc, sout + (int64_t)lane * step);
+      if (S > kWave) {
+        const float *srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
+        for (uint32_t j = lane + kWave; j < S; j += kWave) {
+          sout[(int64_t)j * step] = srow[(int64_t)j * src.dp_xs_stride_elem];
+        }
       }
     }
   }
@@ -379,10 +389,14 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
   if (t >= dispatch_group_tokens(w, tab, g)) return;
+  // The sender of token t inside its DP group (csrc/all_to_all/intranode_dispatch.cu:97).
+  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  RowRegs<NV> regs;
+  load_row<NV, EXACT>(w, src, t, lane, regs);
   const uint32_t slot = lane < w.K ? w.slot_map[(size_t)v * w.K + lane] : kInvalidSlot;
   const uint32_t k0 = part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  fan_out_row<NV, EXACT>(w, tab, g, t, lane, slot, k0, k1, part == 0);
+  store_row<NV, EXACT>(w, tab, src, t, lane, slot, k0, k1, part == 0, regs);
 }
 
 // Small steps: one launch does routing and scatter.  A workgroup owns
@@ -399,6 +413,21 @@ __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint3
   uint32_t *own_slot = ntok + w.G;      // [tokens_per_block][K]
   const uint32_t waves = blockDim.x / kWave;
   const uint32_t tokens_per_block = waves / ksplit;
+
+  // This wave's token.  Its row does not depend on the routing, so the loads go out first
+  // and complete while the workgroup counts; row t exists whenever t < m.
+  const uint32_t lane = lane_id();
+  const uint32_t my_wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t my_j = my_wave / ksplit;
+  const uint32_t my_part = my_wave - my_j * ksplit;
+  const uint32_t my_v = blockIdx.x * tokens_per_block + my_j;
+  const uint32_t my_g = my_v / w.M;
+  const uint32_t my_t = my_v - my_g * w.M;
+  const bool my_in_range = my_j < tokens_per_block && my_g < w.G;
+  const DispatchRank &my_src = tab.at(my_in_range ? my_g * w.dp + my_t % w.dp : 0);
+  const bool my_row_exists = my_in_range && my_t < my_src.m;
+  RowRegs<NV> regs;
+  if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
 
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) hist[e] = 0;
   for (uint32_t g = threadIdx.x; g < w.G; g += blockDim.x) ntok[g] = dispatch_group_tokens(w, tab, g);
@@ -449,19 +478,11 @@ __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint3
     }
   }
 
-  const uint32_t lane = lane_id();
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const uint32_t j = wave / ksplit;
-  const uint32_t part = wave - j * ksplit;
-  const uint32_t v = v0 + j;
-  if (j >= tokens_per_block || v >= total) return;
-  const uint32_t g = v / w.M;
-  const uint32_t t = v - g * w.M;
-  if (t >= ntok[g]) return;
-  const uint32_t slot = lane < w.K ? own_slot[j * w.K + lane] : kInvalidSlot;
-  const uint32_t k0 = part * kper;
+  if (!my_row_exists || my_t >= ntok[my_g]) return;
+  const uint32_t slot = lane < w.K ? own_slot[my_j * w.K + lane] : kInvalidSlot;
+  const uint32_t k0 = my_part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  fan_out_row<NV, EXACT>(w, tab, g, t, lane, slot, k0, k1, part == 0);
+  store_row<NV, EXACT>(w, tab, my_src, my_t, lane, slot, k0, k1, my_part == 0, regs);
 }
 
 // Rows longer than the register variants cover: stream each vector K times.

@@ -388,6 +388,52 @@ def test_geometries(E, K, M, R):
     run_and_check(spec, generate(spec), use_numpy=True)
 
 
+@pytest.mark.parametrize("api", ["world", "per_rank"])
+def test_more_ranks_than_inline_tables_hold(api):
+    """Worlds beyond 64 ranks keep their rank tables in HBM, written by bind kernels."""
+    spec = _small_spec(
+        name="r80", world_size=80, num_experts=160, experts_per_token=4, max_num_tokens=5,
+        hidden_dim=512, in_dtype=FP8,
+    )  # fmt: skip
+    run_and_check(spec, generate(spec), api=api)
+
+
+def test_hbm_tables_under_graph_replay():
+    """A captured step of a > 64-rank world re-binds its tables on every replay, also after
+    eager calls with other tensors have rewritten them."""
+    spec = _small_spec(name="r72-graph", world_size=72, num_experts=72, experts_per_token=2, max_num_tokens=3, hidden_dim=128)
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    other = DeviceStep(spec, generate(spec, seed=9))
+    world = make_world(spec, group_name="r72-graph")
+    stream = torch.cuda.Stream()
+    step.expert_y_all.normal_()
+    other.expert_y_all.normal_()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        step.dispatch_world(world)
+        step.combine_world(world)
+        stream.synchronize()
+        with world.capture() as cap:
+            step.dispatch_world(world)
+            step.combine_world(world)
+        for _ in range(3):
+            other.dispatch_world(world)  # eager step on other tensors in between
+            other.combine_world(world)
+            stream.synchronize()
+            expected_other = check_dispatch_against_oracle(other)
+            check_combine_against_oracle(other, expected_other.slot_map)
+            step.expert_x_all.view(torch.uint8).fill_(0)
+            for t in step.out_tokens:
+                t.fill_(float("nan"))
+            cap.graph.replay(stream)
+            stream.synchronize()
+            expected = check_dispatch_against_oracle(step)
+            check_combine_against_oracle(step, expected.slot_map)
+        cap.graph.destroy()
+    world.destroy()
+
+
 @pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 16384 + 32, 40960])
 def test_row_sizes(hidden_bytes):
     """Rows from one 16-byte vector up to the streaming path for rows beyond 32 KiB."""
