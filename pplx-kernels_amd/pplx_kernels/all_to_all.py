@@ -19,11 +19,13 @@ a world with a single DP group is accepted (the reference asserts
 
 from __future__ import annotations
 
+import sys
 from collections.abc import Callable
 from typing import Any
 
 import torch
 
+from . import ops
 from .ops import _ops
 
 
@@ -41,9 +43,11 @@ class AllToAll:
         self._has_scales = has_scales
 
     def __del__(self) -> None:
+        if sys.is_finalizing():  # the exit hook of pplx_kernels.ops has released everything
+            return
         try:
             self.destroy()
-        except Exception:  # interpreter shutdown: the registry may be gone already
+        except Exception:
             pass
 
     # -- reference API ------------------------------------------------------
@@ -114,7 +118,8 @@ class AllToAll:
     def destroy(self) -> None:
         if self._ptr is not None:
             ptr, self._ptr = self._ptr, None
-            _ops.all_to_all_destroy(ptr)
+            if ops.is_live(ptr):
+                _ops.all_to_all_destroy(ptr)
 
     # -- constructors -------------------------------------------------------
     @classmethod

@@ -16,6 +16,7 @@ the op registration + tensor checks of ``csrc/bindings/all_to_all_ops.cpp:19-24,
 
 from __future__ import annotations
 
+import atexit
 import ctypes
 import os
 import threading
@@ -272,6 +273,29 @@ def _destroy(fptr: int) -> None:
         if not world.handles:
             check_status(lib.pplx_a2a_world_destroy(world.ptr))
             _worlds.pop(world.key, None)
+
+
+def _destroy_all() -> None:
+    """Interpreter exit: release every world while Python and the HIP runtime are still up;
+    AllToAll.__del__ finds nothing left to do afterwards."""
+    try:
+        lib = load_library()
+    except ImportError:
+        return
+    with _registry_lock:
+        for fptr in list(_handle_world):
+            lib.pplx_a2a_destroy(fptr)
+        _handle_world.clear()
+        for world in list(_worlds.values()):
+            lib.pplx_a2a_world_destroy(world.ptr)
+        _worlds.clear()
+
+
+atexit.register(_destroy_all)
+
+
+def is_live(fptr: int) -> bool:
+    return fptr in _handle_world
 
 
 def _create_intranode(

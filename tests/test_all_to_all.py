@@ -202,6 +202,36 @@ def test_all_to_all_reference_flow(in_dtype, out_dtype, internode):
         assert torch.isnan(y[rank_data.num_tokens :]).all()
 
 
+def test_torch_compile_traces_the_ops(backend="inductor"):
+    """use_compile=True of the reference test (tests/test_all_to_all.py:178,262): the ops carry
+    mutating schemas and Meta kernels, so torch.compile (default backend, which mutates the
+    outputs in place) can trace dispatch and combine.  A backend that leaves the ops
+    functionalized would hand them copies of the outputs, which a collective that completes at
+    the last rank's call cannot serve; LoopbackWorld is the entry point for such callers."""
+    import torch._dynamo
+
+    spec = _small_spec(name=f"compile-{backend}", tokens="max")
+    step = DeviceStep(spec, generate(spec))
+    ranks = _make_ranks(spec, f"compile-{backend}")
+    torch._dynamo.reset()
+    try:
+        for r, ata in enumerate(ranks):
+            torch.compile(ata.dispatch, backend=backend)(**_dispatch_kw(step, r))
+    except Exception as exc:  # noqa: BLE001
+        if backend == "inductor" and ("triton" in str(exc).lower() or "inductor" in str(exc).lower()):
+            for a in ranks:
+                a.destroy()
+            pytest.skip(f"inductor unavailable in this image: {str(exc)[:120]}")
+        raise
+    expected = check_dispatch_against_oracle(step)
+    step.expert_y_all.normal_()
+    for r, ata in enumerate(ranks):
+        torch.compile(ata.combine, backend=backend)(**_combine_kw(step, r))
+    check_combine_against_oracle(step, expected.slot_map)
+    for a in ranks:
+        a.destroy()
+
+
 # ---------------------------------------------------------------------------
 # Committed golden vectors through the C ABI
 # ---------------------------------------------------------------------------
