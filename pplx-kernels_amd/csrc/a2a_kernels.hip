@@ -969,6 +969,8 @@ int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipS
     else if (exact && per_lane == 6) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 6, true);                   \
     else if (exact && per_lane == 7) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 7, true);                   \
     else if (exact && per_lane == 8) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 8, true);                   \
+    else if (exact && per_lane == 14) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 14, true);                 \
+    else if (exact && per_lane == 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, true);                 \
     else if (per_lane <= 1) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 1, false);                           \
     else if (per_lane <= 2) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 2, false);                           \
     else if (per_lane <= 4) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 4, false);                           \
@@ -1088,7 +1090,9 @@ bool dispatch_is_fused(const WorldDev &w) {
   // while the whole step's routing is a few tens of KiB.
   const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
   const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
-  return pairs <= kFusedMaxPairs && per_lane <= 8 && (w.E + w.G + 16 * w.K) * 4 <= 48 * 1024;
+  const bool exact = (w.Hb / 16) % kWave == 0;
+  const bool row_fits = per_lane <= 8 || (exact && (per_lane == 14 || per_lane == 16));
+  return pairs <= kFusedMaxPairs && row_fits && (w.E + w.G + 16 * w.K) * 4 <= 48 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {
@@ -1126,7 +1130,9 @@ int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const Disp
   int err = launch_route_t<DT, true>(w, tab, span, s);
   if (err) return err;
   const uint32_t lds = 0;
-  if ((w.Hb / 16 + kWave - 1) / kWave > 8) {
+  const uint32_t per_lane_rows = (w.Hb / 16 + kWave - 1) / kWave;
+  const bool exact_rows = (w.Hb / 16) % kWave == 0;
+  if (per_lane_rows > 8 && !(exact_rows && (per_lane_rows == 14 || per_lane_rows == 16))) {
     hipLaunchKernelGGL(split_pack_long<DT>, dim3(w.M), dim3(256), 0, s, w, tab, g, member, sp);
     return (int)hipGetLastError();
   }
@@ -1152,10 +1158,18 @@ int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const Disp
     if (err != hipSuccess) return (int)err;
   }
   const uint32_t lds = 0;
-  // enough row groups that a hot expert's run is shared by many workgroups
-  const uint32_t spread = w.M >= 2048 ? 16 : w.M >= 256 ? 4 : 1;
+  // Row groups per (local expert, group) run: enough workgroups to cover the CUs even with few
+  // experts per rank, and a hot expert's long run is shared; never more than the run can use.
+  const uint32_t runs = w.L * w.G;
+  uint32_t spread = (2048 + runs - 1) / runs;
+  const uint32_t most = (w.M + 3) / 4;
+  if (spread > most) spread = most;
+  if (spread > 256) spread = 256;
+  if (spread < 1) spread = 1;
   const dim3 grid(w.L * w.G, spread), block(256);
-  if ((w.Hb / 16 + kWave - 1) / kWave > 8) {
+  const uint32_t per_lane_rows = (w.Hb / 16 + kWave - 1) / kWave;
+  const bool exact_rows = (w.Hb / 16) % kWave == 0;
+  if (per_lane_rows > 8 && !(exact_rows && (per_lane_rows == 14 || per_lane_rows == 16))) {
     hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, rank, sp);
     return (int)hipGetLastError();
   }

@@ -18,7 +18,7 @@ ORACLE_LIB = os.path.join(ROOT, "oracle", "liba2a_oracle.so")
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
-    if not os.path.exists(LIB):
+    if not os.path.exists(LIB) or not os.path.exists(os.path.join(ROOT, "pplx-kernels_amd", "bin", "test_a2a")):
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "pplx-kernels_amd", "csrc"), "-s"])
     if not os.path.exists(ORACLE_LIB):
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "-s"])
