@@ -319,44 +319,51 @@ __device__ __forceinline__ void load_row(const WorldDev &w, const DispatchRank &
   }
 }
 
-// Second half: lane k resolves the destination of pick k from `slot`, then the row is stored
-// for picks [k0, k1).
-template <int NV, bool EXACT, class DT>
-__device__ __forceinline__ void store_row(const WorldDev &w, const DT &tab, const DispatchRank &src,
-                                          uint32_t t, uint32_t lane, uint32_t slot, uint32_t k0,
-                                          uint32_t k1, bool report, RowRegs<NV> &regs) {
-  const uint32_t nvec = w.Hb / 16;
-  const uint32_t S = w.S;
-  uint64_t dst_row = 0, dst_scale = 0;
-  int64_t dst_scale_step = 0;
-  if (lane < w.K) {
-    const uint32_t e = src.indices[(size_t)t * w.K + lane];
-    if (e < w.E && slot != kInvalidSlot) {
-      const DispatchRank &dst = tab.at(e / w.L);
-      const uint32_t el = e % w.L;
-      if (slot < dst.x_rows) {
-        dst_row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
-                                             (int64_t)slot * dst.x_stride_row);
-        if (S) {
-          dst_scale = reinterpret_cast<uint64_t>(dst.expert_xs + (int64_t)el * dst.xs_stride_expert +
-                                                 (int64_t)slot * dst.xs_stride_row);
-          dst_scale_step = dst.xs_stride_elem;
-        }
-      } else if (report) {
-        atomicOr(w.faults, kFaultRowDropped);
+// Where pick (expert e, row `slot`) of a token lands: row address, scale-row address and the
+// element stride of the scale row; all zero when the pick has no destination.
+struct Destination {
+  uint64_t row = 0, scale = 0;
+  int64_t scale_step = 0;
+};
+
+template <class DT>
+__device__ __forceinline__ Destination resolve_destination(const WorldDev &w, const DT &tab, uint32_t e,
+                                                           uint32_t slot, bool report) {
+  Destination d;
+  if (e < w.E && slot != kInvalidSlot) {
+    const DispatchRank &dst = tab.at(e / w.L);
+    const uint32_t el = e % w.L;
+    if (slot < dst.x_rows) {
+      d.row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
+                                         (int64_t)slot * dst.x_stride_row);
+      if (w.S) {
+        d.scale = reinterpret_cast<uint64_t>(dst.expert_xs + (int64_t)el * dst.xs_stride_expert +
+                                             (int64_t)slot * dst.xs_stride_row);
+        d.scale_step = dst.xs_stride_elem;
       }
+    } else if (report) {
+      atomicOr(w.faults, kFaultRowDropped);
     }
   }
+  return d;
+}
 
+// Second half: lane k holds the destination of pick k; the row is stored for picks [k0, k1).
+template <int NV, bool EXACT>
+__device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank &src, uint32_t t,
+                                          uint32_t lane, Destination dst, uint32_t k0, uint32_t k1,
+                                          RowRegs<NV> &regs) {
+  const uint32_t nvec = w.Hb / 16;
+  const uint32_t S = w.S;
 #pragma unroll
   for (int i = 0; i < NV; ++i) settle(regs.x[i]);
   settle(regs.sc);
-  settle(dst_row);
-  settle(dst_scale);
-  settle(dst_scale_step);
+  settle(dst.row);
+  settle(dst.scale);
+  settle(dst.scale_step);
 
   for (uint32_t k = k0; k < k1; ++k) {
-    const uint64_t p = read_lane64(dst_row, k);
+    const uint64_t p = read_lane64(dst.row, k);
     if (p == 0) continue;
     PPLX_GLOBAL u32x4 *out = global_ptr<u32x4>(p);
 #pragma unroll
@@ -365,8 +372,8 @@ __device__ __forceinline__ void store_row(const WorldDev &w, const DT &tab, cons
       if (EXACT || j < nvec) __builtin_nontemporal_store(regs.x[i], out + j);
     }
     if (S) {
-      PPLX_GLOBAL float *sout = global_ptr<float>(read_lane64(dst_scale, k));
-      const int64_t step = (int64_t)read_lane64((uint64_t)dst_scale_step, k);
+      PPLX_GLOBAL float *sout = global_ptr<float>(read_lane64(dst.scale, k));
+      const int64_t step = (int64_t)read_lane64((uint64_t)dst.scale_step, k);
       if (lane < S) __builtin_nontemporal_store(regs.sc, sout + (int64_t)lane * step);
       if (S > kWave) {
         const float *srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
@@ -393,48 +400,73 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
   RowRegs<NV> regs;
   load_row<NV, EXACT>(w, src, t, lane, regs);
-  const uint32_t slot = lane < w.K ? w.slot_map[(size_t)v * w.K + lane] : kInvalidSlot;
+  Destination dst;
+  if (lane < w.K) {
+    dst = resolve_destination(w, tab, src.indices[(size_t)t * w.K + lane], w.slot_map[(size_t)v * w.K + lane],
+                              part == 0);
+  }
   const uint32_t k0 = part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  store_row<NV, EXACT>(w, tab, src, t, lane, slot, k0, k1, part == 0, regs);
+  store_row<NV, EXACT>(w, src, t, lane, dst, k0, k1, regs);
 }
 
-// Small steps: one launch does routing and scatter.  A workgroup owns
-// tokens_per_block consecutive virtual tokens.  It first counts, per expert, the
-// picks of all tokens before its own (every workgroup repeats this over the
-// indices, which are a few KiB in L2), then assigns its own tokens' slots in
-// order, then fans the rows out.  The last workgroup has counted everything
-// and writes out_expert_num_tokens.
+// Small steps: one launch does routing and scatter.  A workgroup owns tokens_per_block
+// consecutive virtual tokens and their tokens_per_block * K picks, one thread per pick.
+//   1. every wave issues the loads of its token's row, every pick thread the load of its
+//      expert id: nothing here depends on the routing, so it overlaps with it;
+//   2. the workgroup counts, per expert, the picks of all tokens before its own (every
+//      workgroup repeats this over the indices, which are a few KiB in L2);
+//   3. the pick threads take their slots token by token out of the LDS counters, resolve the
+//      destination rows once for the workgroup and leave them in LDS;
+//   4. the waves fan their rows out.  The last workgroup has counted everything and writes
+//      out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
-  extern __shared__ uint32_t lds_u32[];
-  uint32_t *hist = lds_u32;             // [E]
-  uint32_t *ntok = hist + w.E;          // [G]
-  uint32_t *own_slot = ntok + w.G;      // [tokens_per_block][K]
+  extern __shared__ unsigned long long lds_u64[];
   const uint32_t waves = blockDim.x / kWave;
   const uint32_t tokens_per_block = waves / ksplit;
+  const uint32_t own_pairs = tokens_per_block * w.K;
+  unsigned long long *dst_row = lds_u64;                         // [own_pairs]
+  unsigned long long *dst_scale = dst_row + own_pairs;           // [own_pairs]
+  long long *dst_step = reinterpret_cast<long long *>(dst_scale + own_pairs);  // [own_pairs]
+  uint32_t *hist = reinterpret_cast<uint32_t *>(dst_step + own_pairs);         // [E]
+  uint32_t *ntok = hist + w.E;                                                 // [G]
 
-  // This wave's token.  Its row does not depend on the routing, so the loads go out first
-  // and complete while the workgroup counts; row t exists whenever t < m.
+  const uint32_t total = w.G * w.M;
+  const uint32_t v0 = blockIdx.x * tokens_per_block;
+
+  // 1a. this wave's token and its row
   const uint32_t lane = lane_id();
   const uint32_t my_wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const uint32_t my_j = my_wave / ksplit;
   const uint32_t my_part = my_wave - my_j * ksplit;
-  const uint32_t my_v = blockIdx.x * tokens_per_block + my_j;
+  const uint32_t my_v = v0 + my_j;
   const uint32_t my_g = my_v / w.M;
   const uint32_t my_t = my_v - my_g * w.M;
-  const bool my_in_range = my_j < tokens_per_block && my_g < w.G;
+  const bool my_in_range = my_j < tokens_per_block && my_v < total;
   const DispatchRank &my_src = tab.at(my_in_range ? my_g * w.dp + my_t % w.dp : 0);
   const bool my_row_exists = my_in_range && my_t < my_src.m;
   RowRegs<NV> regs;
   if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
 
+  // 1b. this thread's pick (threads beyond own_pairs have none)
+  const uint32_t pick_j = threadIdx.x / w.K;
+  const uint32_t pick_k = threadIdx.x - pick_j * w.K;
+  const uint32_t pick_v = v0 + pick_j;
+  const uint32_t pick_g = pick_v / w.M;
+  const uint32_t pick_t = pick_v - pick_g * w.M;
+  bool pick_exists = threadIdx.x < own_pairs && pick_v < total;
+  uint32_t pick_e = w.E;
+  if (pick_exists) {
+    const DispatchRank &src = tab.at(pick_g * w.dp + pick_t % w.dp);
+    pick_exists = pick_t < src.m;
+    if (pick_exists) pick_e = src.indices[(size_t)pick_t * w.K + pick_k];
+  }
+
+  // 2. picks of all earlier tokens
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) hist[e] = 0;
   for (uint32_t g = threadIdx.x; g < w.G; g += blockDim.x) ntok[g] = dispatch_group_tokens(w, tab, g);
   __syncthreads();
-
-  const uint32_t v0 = blockIdx.x * tokens_per_block;
-  bool bad_expert = false;
   for (uint32_t v = threadIdx.x; v < v0; v += blockDim.x) {
     const uint32_t g = v / w.M;
     const uint32_t t = v - g * w.M;
@@ -448,41 +480,47 @@ __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint3
   }
   __syncthreads();
 
-  const uint32_t total = w.G * w.M;
+  // 3. own slots, token by token (the experts of one token are distinct: no two threads of a
+  // round share a counter), then the destinations
+  const bool pick_live = pick_exists && pick_t < ntok[pick_g];
+  uint32_t pick_slot = kInvalidSlot;
   for (uint32_t j = 0; j < tokens_per_block; ++j) {
-    const uint32_t v = v0 + j;
-    if (v < total && threadIdx.x < w.K) {
-      const uint32_t g = v / w.M;
-      const uint32_t t = v - g * w.M;
-      uint32_t slot = kInvalidSlot;
-      if (t < ntok[g]) {
-        const uint32_t e = tab.at(g * w.dp + t % w.dp).indices[(size_t)t * w.K + threadIdx.x];
-        if (e < w.E) {
-          slot = hist[e];  // experts of one token are distinct: no two threads share e
-          hist[e] = slot + 1;
-        } else {
-          bad_expert = true;
-        }
-        w.slot_map[(size_t)v * w.K + threadIdx.x] = slot;
-      }
-      own_slot[j * w.K + threadIdx.x] = slot;
+    if (pick_live && pick_j == j && pick_e < w.E) {
+      pick_slot = hist[pick_e];
+      hist[pick_e] = pick_slot + 1;
     }
     __syncthreads();
   }
-  if (bad_expert) atomicOr(w.faults, kFaultBadExpert);
-
+  if (threadIdx.x < own_pairs) {
+    Destination d;
+    if (pick_live) {
+      d = resolve_destination(w, tab, pick_e, pick_slot, true);
+      w.slot_map[(size_t)pick_v * w.K + pick_k] = pick_slot;
+      if (pick_e >= w.E) atomicOr(w.faults, kFaultBadExpert);
+    }
+    dst_row[threadIdx.x] = d.row;
+    dst_scale[threadIdx.x] = d.scale;
+    dst_step[threadIdx.x] = d.scale_step;
+  }
   if (blockIdx.x == gridDim.x - 1) {
     for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
       const DispatchRank &owner = tab.at(e / w.L);
       owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
     }
   }
+  __syncthreads();
 
+  // 4. fan out
   if (!my_row_exists || my_t >= ntok[my_g]) return;
-  const uint32_t slot = lane < w.K ? own_slot[my_j * w.K + lane] : kInvalidSlot;
+  Destination dst;
+  if (lane < w.K) {
+    dst.row = dst_row[my_j * w.K + lane];
+    dst.scale = dst_scale[my_j * w.K + lane];
+    dst.scale_step = dst_step[my_j * w.K + lane];
+  }
   const uint32_t k0 = my_part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  store_row<NV, EXACT>(w, tab, my_src, my_t, lane, slot, k0, k1, my_part == 0, regs);
+  store_row<NV, EXACT>(w, my_src, my_t, lane, dst, k0, k1, regs);
 }
 
 // Rows longer than the register variants cover: stream each vector K times.
@@ -980,6 +1018,10 @@ int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipS
 
 // Number of waves a row's K copies are spread over: few tokens -> more waves,
 // so that the launch still covers the 256 CUs (the row re-reads hit L2).
+uint32_t fused_lds_bytes(const WorldDev &w, uint32_t tokens_per_block) {
+  return tokens_per_block * w.K * 24u + (w.E + w.G) * (uint32_t)sizeof(uint32_t);
+}
+
 uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
   const uint64_t tokens = (uint64_t)w.G * w.M;
   uint32_t ksplit = 1;
@@ -1019,7 +1061,7 @@ int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
   const uint32_t tokens_per_block = kWaves / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
-  const uint32_t lds = (w.E + w.G + tokens_per_block * w.K) * sizeof(uint32_t);
+  const uint32_t lds = fused_lds_bytes(w, tokens_per_block);
 #define PPLX_ROW_KERNEL_ARGS ksplit, kper
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
@@ -1092,7 +1134,7 @@ bool dispatch_is_fused(const WorldDev &w) {
   const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
   const bool exact = (w.Hb / 16) % kWave == 0;
   const bool row_fits = per_lane <= 8 || (exact && (per_lane == 14 || per_lane == 16));
-  return pairs <= kFusedMaxPairs && row_fits && (w.E + w.G + 16 * w.K) * 4 <= 48 * 1024;
+  return pairs <= kFusedMaxPairs && row_fits && 16 * w.K * 24 + (w.E + w.G) * 4 <= 48 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {
