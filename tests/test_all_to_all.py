@@ -686,6 +686,46 @@ def test_graph_replay_decode_shape():
     world.destroy()
 
 
+def test_torch_cuda_graph_with_per_rank_calls():
+    """The reference's "CUDA graph support" as a torch user meets it: torch.cuda.graph around
+    the per-rank AllToAll calls, replayed with new inputs and a new bound_m."""
+    spec = _small_spec(name="torch-graph", in_dtype=FP8, hidden_dim=1024, tokens="uniform")
+    groups = generate(spec)
+    step = DeviceStep(spec, groups)
+    ranks = _make_ranks(spec, "torch-graph")
+    step.expert_y_all.normal_()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):  # warm-up on a side stream, as torch recommends
+        step.dispatch_per_rank(ranks)
+        step.combine_per_rank(ranks)
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step.dispatch_per_rank(ranks)
+        step.combine_per_rank(ranks)
+    for it in range(3):
+        new = generate(spec, seed=50 + it)
+        for r in range(spec.world_size):
+            g = new[r // spec.dp_size]
+            step.dp_x[r].copy_(g.x.cuda())
+            step.dp_x_scale[r].copy_(g.x_scale.cuda())
+            step.indices[r].copy_(g.indices.cuda().to(torch.uint32))
+            step.weights[r].copy_(g.weights.cuda())
+            step.bound_m[r].copy_(torch.tensor([g.n], dtype=torch.uint32).cuda())
+            step.out_tokens[r].fill_(float("nan"))
+        step.groups = new
+        graph.replay()
+        torch.cuda.synchronize()
+        expected = check_dispatch_against_oracle(step)
+        check_combine_against_oracle(step, expected.slot_map)
+        (step.expert_y_all.float().abs().sum() + 1).item()  # eager work between replays
+    del graph
+    for a in ranks:
+        a.destroy()
+
+
 # ---------------------------------------------------------------------------
 # Error behaviour
 # ---------------------------------------------------------------------------
