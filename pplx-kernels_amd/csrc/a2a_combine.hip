@@ -1,0 +1,231 @@
+// gfx950 combine kernel of the MoE dispatch / combine path: the top-k weighted
+// gather-reduce, for expert_y in place (one-call mode) or for the staged rows of split mode.
+#include "a2a_common.h"
+
+namespace pplx_amd {
+namespace {
+
+// ---------------------------------------------------------------------------
+// Combine: out[t, :] = (U) sum_k w[t, k] * (float) expert_y[e_k][slot(t, k), :]
+// with k ascending and fp32 accumulation
+// (csrc/all_to_all/intranode_combine.cu:141-168).
+// ---------------------------------------------------------------------------
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+  struct Raw {
+    f32x4 a, b;
+  };
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
+    const PPLX_GLOBAL f32x4 *p = global_cptr<f32x4>(row) + 2 * (size_t)vec;
+    return Raw{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1)};
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &r) {
+    return __builtin_shufflevector(r.a, r.b, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+  // N rows held as 2 N registers of 16 bytes
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) {
+    SettleAll<2 * N>::of(reinterpret_cast<f32x4 *>(raw));
+  }
+};
+template <> struct Row8<__bf16> {
+  typedef u32x4 Raw;
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
+    return __builtin_nontemporal_load(global_cptr<u32x4>(row) + vec);
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
+    f32x8 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = __uint_as_float(raw[i] << 16);
+      out[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+    }
+    return out;
+  }
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) { SettleAll<N>::of(raw); }
+};
+template <> struct Row8<_Float16> {
+  typedef f16x8 Raw;
+  static __device__ __forceinline__ Raw load(uint64_t row, uint32_t vec) {
+    return __builtin_nontemporal_load(global_cptr<f16x8>(row) + vec);
+  }
+  static __device__ __forceinline__ f32x8 widen(const Raw &raw) {
+    return __builtin_convertvector(raw, f32x8);
+  }
+  template <int N> static __device__ __forceinline__ void settle(Raw *raw) { SettleAll<N>::of(raw); }
+};
+
+template <typename U> struct Store8;
+template <> struct Store8<__bf16> {
+  static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
+    __builtin_nontemporal_store(__builtin_convertvector(acc, bf16x8), reinterpret_cast<bf16x8 *>(row) + vec);
+  }
+};
+template <> struct Store8<_Float16> {
+  static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
+    __builtin_nontemporal_store(__builtin_convertvector(acc, f16x8), reinterpret_cast<f16x8 *>(row) + vec);
+  }
+};
+
+// N picks starting at k: all N loads are issued before the first is used.
+template <typename T, int N>
+__device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, float weight_of_lane,
+                                             uint32_t k, uint32_t vec) {
+  typename Row8<T>::Raw raw[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) raw[i] = Row8<T>::load(read_lane64(row_of_lane, k + i), vec);
+  Row8<T>::template settle<N>(raw);
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float wk = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight_of_lane), (int)(k + i)));
+    acc += wk * Row8<T>::widen(raw[i]);
+  }
+}
+
+// One wave owns VPL * 64 consecutive 8-element vectors of one output row.  With
+// KK == 0 (any K) it is one vector per lane and the picks go in groups of up to
+// eight loads; with KK in {1, 2, 4} the wave takes VPL = 8 / KK vectors per lane so
+// that eight row loads per lane are in flight for small top-k too.
+template <typename T, typename U, class CT, int KK, int VPL>
+__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments,
+                                                      uint32_t first_rank, uint32_t rank_count,
+                                                      const uint8_t *stage_y, uint64_t stage_row_bytes) {
+  const uint32_t lane = lane_id();
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
+                                                       threadIdx.x / kWave);
+  const uint32_t token = wave / segments;
+  const uint32_t segment = wave - token * segments;
+  const uint32_t r_local = token / w.M;
+  const uint32_t t = token - r_local * w.M;
+  if (r_local >= rank_count) return;
+  const uint32_t r = first_rank + r_local;
+  const CombineRank &c = tab.at(r);
+  if (t >= combine_rank_tokens(w, c)) return;
+
+  // Lane k resolves pick k: no LDS, no barrier.
+  uint64_t row = 0;
+  float weight = 0.f;
+  if (lane < w.K) {
+    const uint32_t e = c.indices[(size_t)t * w.K + lane];
+    const uint32_t slot = w.slot_map[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
+    weight = c.weights[(int64_t)t * c.w_stride_row + lane];
+    if (CT::kStaged) {
+      // combine SEND left the row of (token, pick) in the staging area.
+      if (e < w.E && slot != kInvalidSlot) {
+        row = reinterpret_cast<uint64_t>(stage_y) +
+              (((uint64_t)(r / w.dp) * w.M + t) * w.K + lane) * stage_row_bytes;
+      }
+    } else if (e < w.E && slot != kInvalidSlot) {
+      const CombineRank &owner = tab.at(e / w.L);
+      if (slot < owner.y_rows) {
+        row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
+                                         (int64_t)(e % w.L) * owner.y_stride_expert +
+                                         (int64_t)slot * owner.y_stride_row);
+      } else if (segment == 0) {
+        atomicOr(w.faults, kFaultBadSlot);
+      }
+    }
+  }
+  const bool all_rows = __builtin_amdgcn_ballot_w64(lane < w.K && row == 0) == 0;
+
+  U *out = reinterpret_cast<U *>(c.out_tokens) + (int64_t)t * c.out_stride_row;
+  const uint32_t nvec = w.H / 8;
+  const uint32_t K = w.K;
+  if (!all_rows) {
+    // A pick without a row (bad expert id or slot) contributes nothing.
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
+      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (uint32_t k = 0; k < K; ++k) {
+        if (read_lane64(row, k) != 0) gather_group<T, 1>(acc, row, weight, k, vec_ld);
+      }
+      if (vec < nvec) Store8<U>::at(out, vec, acc);
+    }
+    return;
+  }
+  if (KK == 0) {
+    const uint32_t vec = segment * kWave + lane;
+    const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;  // clamp: loads stay unconditional
+    f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint32_t k = 0;
+    for (; k + 8 <= K; k += 8) gather_group<T, 8>(acc, row, weight, k, vec_ld);
+    if (K & 4) { gather_group<T, 4>(acc, row, weight, k, vec_ld); k += 4; }
+    if (K & 2) { gather_group<T, 2>(acc, row, weight, k, vec_ld); k += 2; }
+    if (K & 1) { gather_group<T, 1>(acc, row, weight, k, vec_ld); }
+    if (vec < nvec) Store8<U>::at(out, vec, acc);
+  } else {
+    constexpr int N = KK == 0 ? 1 : KK;
+    typename Row8<T>::Raw raw[VPL][N];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
+#pragma unroll
+      for (int k = 0; k < N; ++k) raw[v][k] = Row8<T>::load(read_lane64(row, k), vec_ld);
+    }
+    Row8<T>::template settle<VPL * N>(&raw[0][0]);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const uint32_t vec = (segment * VPL + v) * kWave + lane;
+      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        const float wk = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), k));
+        acc += wk * Row8<T>::widen(raw[v][k]);
+      }
+      if (vec < nvec) Store8<U>::at(out, vec, acc);
+    }
+  }
+}
+
+template <typename T, typename U, class CT>
+int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
+                     const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
+  const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
+  const uint32_t vpl = w.K == 1 ? 8 : w.K == 2 ? 4 : w.K == 4 ? 2 : 1;
+  const uint32_t segments = (nvec_segments + vpl - 1) / vpl;
+  const uint64_t waves = (uint64_t)rank_count * w.M * segments;
+  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
+  switch (w.K) {
+    case 1: hipLaunchKernelGGL((combine_gather<T, U, CT, 1, 8>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    case 2: hipLaunchKernelGGL((combine_gather<T, U, CT, 2, 4>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    case 4: hipLaunchKernelGGL((combine_gather<T, U, CT, 4, 2>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+    default: hipLaunchKernelGGL((combine_gather<T, U, CT, 0, 1>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+  }
+  return (int)hipGetLastError();
+}
+
+template <class CT>
+int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s,
+                     uint32_t first_rank, uint32_t rank_count, const uint8_t *stage_y = nullptr,
+                     uint64_t stage_row_bytes = 0) {
+  // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
+  switch (in_dtype * 4 + out_dtype) {
+    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
+                              uint32_t rank, int in_dtype, int out_dtype, void *stream) {
+  return launch_combine_t(w, SingleCombine{row}, in_dtype, out_dtype, (hipStream_t)stream, rank, 1,
+                          sp.stage_y, sp.y_row_bytes);
+}
+
+int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
+                   void *stream) {
+  if (inline_rows)
+    return launch_combine_t(w, make_inline(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream, 0, w.R);
+  return launch_combine_t(w, HbmCombine{w.crank}, in_dtype, out_dtype, (hipStream_t)stream, 0, w.R);
+}
+
+}  // namespace pplx_amd

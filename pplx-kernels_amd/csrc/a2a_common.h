@@ -1,0 +1,140 @@
+// Device-side helpers shared by the kernel sources of the dispatch / combine path:
+// vector types, the rank-table flavours a kernel can be instantiated for, address-space
+// casts, scheduling barriers and wave utilities.  Included only by the .hip sources; every
+// definition sits in an unnamed namespace of the including translation unit.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "a2a_device.h"
+
+namespace pplx_amd {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+struct InlineDispatch {
+  DispatchRank rows[kInlineRanks];
+  __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
+};
+struct HbmDispatch {
+  const DispatchRank *rows;
+  __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
+};
+struct InlineCombine {
+  static constexpr bool kStaged = false;
+  CombineRank rows[kInlineRanks];
+  __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
+};
+struct HbmCombine {
+  static constexpr bool kStaged = false;
+  const CombineRank *rows;
+  __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
+};
+
+// Pointers rebuilt from integers would be "flat" to the compiler; these casts say
+// that they are global memory, so that plain global_load / global_store are emitted.
+#define PPLX_GLOBAL __attribute__((address_space(1)))
+template <typename V>
+__device__ __forceinline__ PPLX_GLOBAL V *global_ptr(uint64_t address) {
+  return (PPLX_GLOBAL V *)address;
+}
+template <typename V>
+__device__ __forceinline__ const PPLX_GLOBAL V *global_cptr(uint64_t address) {
+  return (const PPLX_GLOBAL V *)address;
+}
+
+// Makes the compiler treat `v` as consumed here, so that it waits for the loads
+// feeding it at this point and not inside a later loop, where such a wait would
+// also drain the stores of the previous iteration.
+template <typename V>
+__device__ __forceinline__ void settle(V &v) {
+  asm volatile("" : "+v"(v));
+}
+
+// settle() for N registers at once: every load feeding them has to be issued
+// before this point, so the N loads go out back to back behind one wait.
+template <int N> struct SettleAll;
+template <> struct SettleAll<1> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) { asm volatile("" : "+v"(r[0])); }
+};
+template <> struct SettleAll<2> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]));
+  }
+};
+template <> struct SettleAll<4> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+  }
+};
+template <> struct SettleAll<8> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile(""
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
+                   "+v"(r[7]));
+  }
+};
+template <> struct SettleAll<16> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile(""
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
+                   "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]),
+                   "+v"(r[13]), "+v"(r[14]), "+v"(r[15]));
+  }
+};
+
+// Split mode: a launch sees only the calling rank's arguments (its peers may not
+// have called yet), whatever rank index is asked for.
+struct SingleDispatch {
+  DispatchRank row;
+  __device__ __forceinline__ const DispatchRank &at(uint32_t) const { return row; }
+};
+struct SingleCombine {
+  static constexpr bool kStaged = true;  // rows come from the world's stage_y, not expert_y
+  CombineRank row;
+  __device__ __forceinline__ const CombineRank &at(uint32_t) const { return row; }
+};
+
+__device__ __forceinline__ uint32_t lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+__device__ __forceinline__ uint64_t read_lane64(uint64_t v, uint32_t src_lane) {
+  return ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), (int)src_lane) << 32) |
+         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, (int)src_lane);
+}
+
+// Tokens present in DP group g this step: the reference's numSendTokens
+// (csrc/all_to_all/intranode_dispatch.cu:64), clamped to the rows that exist.
+template <class DT>
+__device__ __forceinline__ uint32_t dispatch_group_tokens(const WorldDev &w, const DT &tab, uint32_t g) {
+  const DispatchRank &r = tab.at(g * w.dp);
+  uint32_t n = r.bound_m ? *r.bound_m : r.m;
+  n = n < r.m ? n : r.m;
+  return n < w.M ? n : w.M;
+}
+
+__device__ __forceinline__ uint32_t combine_rank_tokens(const WorldDev &w, const CombineRank &c) {
+  uint32_t n = c.bound_m ? *c.bound_m : c.m;
+  n = n < c.m ? n : c.m;
+  return n < w.M ? n : w.M;
+}
+
+inline InlineDispatch make_inline(const WorldDev &w, const DispatchRank *rows) {
+  InlineDispatch t{};
+  for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
+  return t;
+}
+
+inline InlineCombine make_inline(const WorldDev &w, const CombineRank *rows) {
+  InlineCombine t{};
+  for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
+  return t;
+}
+
+}  // namespace
+}  // namespace pplx_amd

@@ -132,7 +132,8 @@ struct BindCombineBatch {
   CombineRank rows[kBindBatch];
 };
 
-// Launchers implemented in a2a_kernels.hip; they return a hipError_t as int.
+// Launchers implemented in a2a_dispatch.hip, a2a_combine.hip and a2a_split.hip; they return a
+// hipError_t as int.
 // `inline_rows` (world_size rows, host memory) selects the inline-table kernels;
 // NULL selects the HBM tables, which must have been bound.
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream);
