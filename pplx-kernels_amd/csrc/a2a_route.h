@@ -45,7 +45,29 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
   uint32_t *lds_base = reinterpret_cast<uint32_t *>(lds_mask + (size_t)chunks * w.E);
 
   for (uint32_t i = threadIdx.x; i < chunks * w.E; i += blockDim.x) lds_mask[i] = 0ull;
+  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_base[e] = 0;
   __syncthreads();
+
+  // Rows taken by earlier tiles, summed per expert into lds_base[0][e] by the whole workgroup:
+  // the counts are fetched kTileLoads at a time so that their latencies overlap each other and
+  // the index loads below (one thread per expert walking the tiles would pay one L2 round trip
+  // per tile).
+  {
+    constexpr uint32_t kTileLoads = 8;
+    const uint32_t total = blockIdx.x * w.E;
+    for (uint32_t first = threadIdx.x; first < total; first += blockDim.x * kTileLoads) {
+      uint32_t rows[kTileLoads];
+#pragma unroll
+      for (uint32_t u = 0; u < kTileLoads; ++u) {
+        const uint32_t j = first + u * blockDim.x;
+        rows[u] = j < total ? span.tile_cnt[j] : 0u;
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kTileLoads; ++u) {
+        if (rows[u]) atomicAdd(&lds_base[(first + u * blockDim.x) % w.E], rows[u]);
+      }
+    }
+  }
 
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t chunk = threadIdx.x / kWave;
@@ -71,11 +93,10 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
   }
   __syncthreads();
 
-  // Per expert: rows taken by earlier tiles, then running prefix over chunks.
+  // Per expert: running prefix over chunks, starting from the rows of earlier tiles.
   const bool last_tile = blockIdx.x == gridDim.x - 1;
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
-    uint32_t running = 0;
-    for (uint32_t tile = 0; tile < blockIdx.x; ++tile) running += span.tile_cnt[(size_t)tile * w.E + e];
+    uint32_t running = lds_base[e];
     for (uint32_t c = 0; c < chunks; ++c) {
       lds_base[c * w.E + e] = running;
       running += __popcll(lds_mask[(size_t)c * w.E + e]);
