@@ -275,6 +275,16 @@ int flush_table(pplx_a2a_world &w, const std::vector<Row> &rows, std::vector<Row
   return PPLX_A2A_OK;
 }
 
+// Widest load (in expert ids) that suits the indices of every rank of the pending step.
+uint32_t pick_vector_of(const pplx_a2a_world &w) {
+  uint32_t pv = w.dev.K % 4 == 0 ? 4 : w.dev.K % 2 == 0 ? 2 : 1;
+  for (const DispatchRank &r : w.pend_dispatch) {
+    const uintptr_t p = reinterpret_cast<uintptr_t>(r.indices);
+    while (pv > 1 && p % (4 * pv) != 0) pv /= 2;
+  }
+  return pv;
+}
+
 int run_dispatch(pplx_a2a_world &w, void *stream) {
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
@@ -283,14 +293,14 @@ int run_dispatch(pplx_a2a_world &w, void *stream) {
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
   if (w.dev.R <= kInlineRanks) {
-    LAUNCH_TRY(launch_dispatch(w.dev, w.pend_dispatch.data(), stream));
+    LAUNCH_TRY(launch_dispatch(w.dev, w.pend_dispatch.data(), pick_vector_of(w), stream));
     return PPLX_A2A_OK;
   }
   st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
                                                     w.bound_dispatch_valid, false,
                                                     launch_bind_dispatch, stream);
   if (st) return st;
-  LAUNCH_TRY(launch_dispatch(w.dev, nullptr, stream));
+  LAUNCH_TRY(launch_dispatch(w.dev, nullptr, pick_vector_of(w), stream));
   return PPLX_A2A_OK;
 }
 

@@ -17,10 +17,12 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 struct InlineDispatch {
+  static constexpr bool kInline = true;  // the table itself is the kernel argument
   DispatchRank rows[kInlineRanks];
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
 struct HbmDispatch {
+  static constexpr bool kInline = false;
   const DispatchRank *rows;
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
@@ -45,6 +47,17 @@ __device__ __forceinline__ PPLX_GLOBAL V *global_ptr(uint64_t address) {
 template <typename V>
 __device__ __forceinline__ const PPLX_GLOBAL V *global_cptr(uint64_t address) {
   return (const PPLX_GLOBAL V *)address;
+}
+// The same for a pointer that was read back from a table (out of LDS or HBM, where the
+// compiler cannot see what it points to): a flat load would also tie up the LDS counter and
+// make every later wait a wait for everything.
+template <typename V>
+__device__ __forceinline__ const PPLX_GLOBAL V *as_global(const V *p) {
+  return (const PPLX_GLOBAL V *)p;
+}
+template <typename V>
+__device__ __forceinline__ PPLX_GLOBAL V *as_global(V *p) {
+  return (PPLX_GLOBAL V *)p;
 }
 
 // Makes the compiler treat `v` as consumed here, so that it waits for the loads
@@ -90,6 +103,7 @@ template <> struct SettleAll<16> {
 // Split mode: a launch sees only the calling rank's arguments (its peers may not
 // have called yet), whatever rank index is asked for.
 struct SingleDispatch {
+  static constexpr bool kInline = false;
   DispatchRank row;
   __device__ __forceinline__ const DispatchRank &at(uint32_t) const { return row; }
 };
@@ -113,13 +127,13 @@ __device__ __forceinline__ uint64_t read_lane64(uint64_t v, uint32_t src_lane) {
 template <class DT>
 __device__ __forceinline__ uint32_t dispatch_group_tokens(const WorldDev &w, const DT &tab, uint32_t g) {
   const DispatchRank &r = tab.at(g * w.dp);
-  uint32_t n = r.bound_m ? *r.bound_m : r.m;
+  uint32_t n = r.bound_m ? *as_global(r.bound_m) : r.m;
   n = n < r.m ? n : r.m;
   return n < w.M ? n : w.M;
 }
 
 __device__ __forceinline__ uint32_t combine_rank_tokens(const WorldDev &w, const CombineRank &c) {
-  uint32_t n = c.bound_m ? *c.bound_m : c.m;
+  uint32_t n = c.bound_m ? *as_global(c.bound_m) : c.m;
   n = n < c.m ? n : c.m;
   return n < w.M ? n : w.M;
 }

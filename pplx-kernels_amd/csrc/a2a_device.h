@@ -138,7 +138,10 @@ struct BindCombineBatch {
 // NULL selects the HBM tables, which must have been bound.
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream);
 int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stream);
-int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *stream);
+// pick_vector: how many expert ids one load may fetch from any rank's indices (4, 2 or 1):
+// K must be a multiple of it and every indices pointer aligned to 4 * pick_vector bytes.
+int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t pick_vector,
+                    void *stream);
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
 // Split mode phases of one rank (`row` holds that rank's arguments of the call).

@@ -69,27 +69,147 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   store_row<NV, EXACT>(w, src, t, lane, dst, k0, k1, regs);
 }
 
+// dispatch_fused always runs with this many threads (16 waves): fewer, larger workgroups
+// repeat less counting, and a compile-time size keeps its first loads free of any wait.
+constexpr uint32_t kFusedThreads = 1024;
+
+// A rank table that dispatch_fused has copied into LDS.
+struct LdsDispatch {
+  const DispatchRank *rows;
+  __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
+};
+
+// PV consecutive expert ids as one register value (PV = 1, 2 or 4).
+template <int PV> struct PickVector;
+template <> struct PickVector<1> {
+  typedef uint32_t type;
+  static __device__ __forceinline__ uint32_t at(type x, int) { return x; }
+};
+template <> struct PickVector<2> {
+  typedef uint32_t type __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
+};
+template <> struct PickVector<4> {
+  typedef u32x4 type;
+  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
+};
+
+// Reads the picks of virtual tokens [0, v_own_end), one thread per token and PV picks per load
+// (K % PV == 0 and every indices pointer aligned to the vector: the host checks both): those
+// of tokens before v_own go into the LDS histogram, those of the workgroup's own tokens
+// [v_own, v_own_end) into own_e for phase 3.
+//
+// The loads of a token (its group's token count and its first two vectors of picks) are
+// unconditional, from a harmless address when the thread has no token, and sit in
+// straight-line code: they are issued together and cost one trip to memory, and the count is
+// applied afterwards.  `between` runs after the loads of the thread's first token have been
+// issued and before they are used: whatever it loads is in flight behind them (a wave's loads
+// complete in order).  The bookkeeping per token is one division: this loop is bound by the
+// ALU, not by memory, when every workgroup of a launch repeats it.
+template <int PV, class Table, class Between>
+__device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows, uint32_t v_own,
+                                           uint32_t v_own_end, uint32_t *hist, uint32_t *own_e,
+                                           Between &&between) {
+  typedef PickVector<PV> Vec;
+  typedef typename Vec::type vec_t;
+  const uint32_t vectors = w.K / PV;
+  struct Fetch {
+    vec_t a, b;           // vectors 0 and 1 of the token's picks (b repeats a when there is one)
+    uint32_t n;           // tokens present in the group
+    uint32_t t;           // token inside its group
+    const PPLX_GLOBAL vec_t *idx;
+    bool valid;
+  };
+  auto issue = [&](uint32_t v) {
+    Fetch f;
+    const bool in_range = v < v_own_end;
+    const uint32_t g = in_range ? v / w.M : 0;
+    f.t = in_range ? v - g * w.M : 0;
+    const DispatchRank &head = rows.at(g * w.dp);
+    const DispatchRank &src = w.dp == 1 ? head : rows.at(g * w.dp + f.t % w.dp);
+    f.valid = in_range && f.t < src.m && f.t < head.m;
+    const bool bounded = f.valid && head.bound_m != nullptr;
+    const uint32_t loaded_n = *as_global(bounded ? head.bound_m : w.faults);
+    f.idx = as_global(reinterpret_cast<const vec_t *>(f.valid ? src.indices + (size_t)f.t * w.K : w.slot_map));
+    f.a = f.idx[0];
+    f.b = f.idx[vectors > 1 ? 1 : 0];
+    f.n = bounded ? loaded_n : head.m;
+    return f;
+  };
+  auto place = [&](uint32_t v, uint32_t j, vec_t a, vec_t b, const Fetch &f) {
+    const bool second = j + 1 < vectors;
+    if (v >= v_own) {
+      uint32_t *keep = own_e + (v - v_own) * w.K + j * PV;
+#pragma unroll
+      for (int u = 0; u < PV; ++u) keep[u] = Vec::at(a, u);
+#pragma unroll
+      for (int u = 0; u < PV; ++u) {
+        if (second) keep[PV + u] = Vec::at(b, u);
+      }
+    } else if (f.t < f.n) {
+#pragma unroll
+      for (int u = 0; u < PV; ++u) {
+        const uint32_t e = Vec::at(a, u);
+        if (e < w.E) atomicAdd(&hist[e], 1u);
+      }
+#pragma unroll
+      for (int u = 0; u < PV; ++u) {
+        const uint32_t e = Vec::at(b, u);
+        if (second && e < w.E) atomicAdd(&hist[e], 1u);
+      }
+    }
+  };
+  auto consume = [&](uint32_t v, const Fetch &f) {
+    if (!f.valid) return;
+    place(v, 0, f.a, f.b, f);
+    for (uint32_t j = 2; j < vectors; j += 2) place(v, j, f.idx[j], f.idx[j + 1 < vectors ? j + 1 : j], f);
+  };
+
+  const Fetch first = issue(threadIdx.x);
+  between();
+  consume(threadIdx.x, first);
+  for (uint32_t v = threadIdx.x + kFusedThreads; v < v_own_end; v += kFusedThreads) consume(v, issue(v));
+}
+
 // Small steps: one launch does routing and scatter.  A workgroup owns tokens_per_block
 // consecutive virtual tokens and their tokens_per_block * K picks, one thread per pick.
-//   1. every wave issues the loads of its token's row, every pick thread the load of its
-//      expert id: nothing here depends on the routing, so it overlaps with it;
-//   2. the workgroup counts, per expert, the picks of all tokens before its own (every
-//      workgroup repeats this over the indices, which are a few KiB in L2);
+//   0. a rank table that came inline is copied from the kernel arguments into LDS with loads
+//      that depend on nothing, so every later lookup is an LDS read and not another trip to
+//      memory behind the one that fetches the geometry;
+//   1. index arithmetic for the wave's token and the thread's pick;
+//   2. the workgroup reads the picks of all tokens up to and including its own and counts, per
+//      expert, those of the tokens before its own (every workgroup repeats this over the
+//      indices, which are a few KiB in L2); then every wave issues the loads of its token's
+//      row, which is needed only in phase 4;
 //   3. the pick threads take their slots token by token out of the LDS counters, resolve the
 //      destination rows once for the workgroup and leave them in LDS;
 //   4. the waves fan their rows out.  The last workgroup has counted everything and writes
 //      out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+__global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper,
+                                                              uint32_t pick_vector) {
   extern __shared__ unsigned long long lds_u64[];
-  const uint32_t waves = blockDim.x / kWave;
+  constexpr bool kStaged = DT::kInline;
+  constexpr uint32_t kTableWords = kStaged ? sizeof(DT) / 8 : 0;
+  if constexpr (kStaged) {
+    const unsigned long long *args = reinterpret_cast<const unsigned long long *>(&tab);
+    for (uint32_t i = threadIdx.x; i < kTableWords; i += kFusedThreads) lds_u64[i] = args[i];
+  }
+  const uint32_t waves = kFusedThreads / kWave;
   const uint32_t tokens_per_block = waves / ksplit;
   const uint32_t own_pairs = tokens_per_block * w.K;
-  unsigned long long *dst_row = lds_u64;                         // [own_pairs]
-  unsigned long long *dst_scale = dst_row + own_pairs;           // [own_pairs]
+  unsigned long long *dst_row = lds_u64 + kTableWords;                         // [own_pairs]
+  unsigned long long *dst_scale = dst_row + own_pairs;                         // [own_pairs]
   long long *dst_step = reinterpret_cast<long long *>(dst_scale + own_pairs);  // [own_pairs]
   uint32_t *hist = reinterpret_cast<uint32_t *>(dst_step + own_pairs);         // [E]
   uint32_t *ntok = hist + w.E;                                                 // [G]
+  uint32_t *own_e = ntok + w.G;                                                // [own_pairs]
+  for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) hist[e] = 0;
+  if constexpr (kStaged) __syncthreads();
+  const LdsDispatch staged{reinterpret_cast<const DispatchRank *>(lds_u64)};
+  auto rows = [&]() -> decltype(auto) {
+    if constexpr (kStaged) return (staged); else return (tab);
+  };
 
   const uint32_t total = w.G * w.M;
   const uint32_t v0 = blockIdx.x * tokens_per_block;
@@ -103,10 +223,8 @@ __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint3
   const uint32_t my_g = my_v / w.M;
   const uint32_t my_t = my_v - my_g * w.M;
   const bool my_in_range = my_j < tokens_per_block && my_v < total;
-  const DispatchRank &my_src = tab.at(my_in_range ? my_g * w.dp + my_t % w.dp : 0);
+  const DispatchRank &my_src = rows().at(my_in_range ? my_g * w.dp + my_t % w.dp : 0);
   const bool my_row_exists = my_in_range && my_t < my_src.m;
-  RowRegs<NV> regs;
-  if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
 
   // 1b. this thread's pick (threads beyond own_pairs have none)
   const uint32_t pick_j = threadIdx.x / w.K;
@@ -115,59 +233,71 @@ __global__ __launch_bounds__(1024) void dispatch_fused(WorldDev w, DT tab, uint3
   const uint32_t pick_g = pick_v / w.M;
   const uint32_t pick_t = pick_v - pick_g * w.M;
   bool pick_exists = threadIdx.x < own_pairs && pick_v < total;
-  uint32_t pick_e = w.E;
-  if (pick_exists) {
-    const DispatchRank &src = tab.at(pick_g * w.dp + pick_t % w.dp);
-    pick_exists = pick_t < src.m;
-    if (pick_exists) pick_e = src.indices[(size_t)pick_t * w.K + pick_k];
-  }
+  if (pick_exists) pick_exists = pick_t < rows().at(pick_g * w.dp + pick_t % w.dp).m;
 
   // 2. picks of all earlier tokens
-  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) hist[e] = 0;
-  for (uint32_t g = threadIdx.x; g < w.G; g += blockDim.x) ntok[g] = dispatch_group_tokens(w, tab, g);
-  __syncthreads();
-  for (uint32_t v = threadIdx.x; v < v0; v += blockDim.x) {
-    const uint32_t g = v / w.M;
-    const uint32_t t = v - g * w.M;
-    if (t < ntok[g]) {
-      const uint32_t *idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
-      for (uint32_t k = 0; k < w.K; ++k) {
-        const uint32_t e = idx[k];
-        if (e < w.E) atomicAdd(&hist[e], 1u);
-      }
-    }
+  // (the token count of group `threadIdx.x` is fetched ahead of the picks, in the same batch of
+  // loads, and stored once they have been used: no wave pays for two trips to memory in a row)
+  const bool counts_group = threadIdx.x < w.G;
+  const DispatchRank &counted = rows().at(counts_group ? threadIdx.x * w.dp : 0);
+  const uint32_t *counted_bound = counts_group ? counted.bound_m : nullptr;
+  const uint32_t counted_loaded = *as_global(counted_bound ? counted_bound : w.faults);
+  const uint32_t v_own_end = v0 + tokens_per_block < total ? v0 + tokens_per_block : total;
+  // The row is fetched behind the first picks: a wave's loads complete in order, so the small
+  // loads would otherwise wait behind several KiB of row data.  It is needed in phase 4.
+  RowRegs<NV> regs;
+  auto fetch_row = [&]() {
+    if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
+  };
+  if (pick_vector == 4) {
+    read_picks<4>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+  } else if (pick_vector == 2) {
+    read_picks<2>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+  } else {
+    read_picks<1>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+  }
+  if (counts_group) {
+    uint32_t n = counted_bound ? counted_loaded : counted.m;
+    n = n < counted.m ? n : counted.m;
+    ntok[threadIdx.x] = n < w.M ? n : w.M;
+  }
+  for (uint32_t g = threadIdx.x + kFusedThreads; g < w.G; g += kFusedThreads) {
+    ntok[g] = dispatch_group_tokens(w, rows(), g);
   }
   __syncthreads();
 
   // 3. own slots, token by token (the experts of one token are distinct: no two threads of a
   // round share a counter), then the destinations
   const bool pick_live = pick_exists && pick_t < ntok[pick_g];
+  const uint32_t pick_e = pick_exists ? own_e[threadIdx.x] : w.E;
   uint32_t pick_slot = kInvalidSlot;
+  // (when all pick threads sit in one wave its LDS accesses are ordered by themselves)
+  const bool one_wave = own_pairs <= kWave;
   for (uint32_t j = 0; j < tokens_per_block; ++j) {
     if (pick_live && pick_j == j && pick_e < w.E) {
       pick_slot = hist[pick_e];
       hist[pick_e] = pick_slot + 1;
     }
-    __syncthreads();
+    if (!one_wave) __syncthreads();
   }
   if (threadIdx.x < own_pairs) {
     Destination d;
     if (pick_live) {
-      d = resolve_destination(w, tab, pick_e, pick_slot, true);
-      w.slot_map[(size_t)pick_v * w.K + pick_k] = pick_slot;
+      d = resolve_destination(w, rows(), pick_e, pick_slot, true);
+      as_global(w.slot_map)[(size_t)pick_v * w.K + pick_k] = pick_slot;
       if (pick_e >= w.E) atomicOr(w.faults, kFaultBadExpert);
     }
     dst_row[threadIdx.x] = d.row;
     dst_scale[threadIdx.x] = d.scale;
     dst_step[threadIdx.x] = d.scale_step;
   }
+  __syncthreads();
   if (blockIdx.x == gridDim.x - 1) {
-    for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
-      const DispatchRank &owner = tab.at(e / w.L);
-      owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
+    for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) {
+      const DispatchRank &owner = rows().at(e / w.L);
+      as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
     }
   }
-  __syncthreads();
 
   // 4. fan out
   if (!my_row_exists || my_t >= ntok[my_g]) return;
@@ -240,8 +370,9 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab)
 
 // Number of waves a row's K copies are spread over: few tokens -> more waves,
 // so that the launch still covers the 256 CUs (the row re-reads hit L2).
-uint32_t fused_lds_bytes(const WorldDev &w, uint32_t tokens_per_block) {
-  return tokens_per_block * w.K * 24u + (w.E + w.G) * (uint32_t)sizeof(uint32_t);
+uint32_t fused_lds_bytes(const WorldDev &w, uint32_t tokens_per_block, bool inline_table) {
+  const uint32_t table = inline_table ? (uint32_t)sizeof(InlineDispatch) : 0u;
+  return table + tokens_per_block * w.K * 28u + (w.E + w.G) * (uint32_t)sizeof(uint32_t);
 }
 
 uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
@@ -276,15 +407,15 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
 }
 
 template <class DT>
-int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
-  constexpr uint32_t kWaves = 16;  // 1024 threads: fewer, larger workgroups repeat less counting
+  constexpr uint32_t kWaves = kFusedThreads / kWave;
   const uint32_t ksplit = pick_ksplit(w, kWaves);
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
   const uint32_t tokens_per_block = kWaves / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
-  const uint32_t lds = fused_lds_bytes(w, tokens_per_block);
-#define PPLX_ROW_KERNEL_ARGS ksplit, kper
+  const uint32_t lds = fused_lds_bytes(w, tokens_per_block, DT::kInline);
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper, pick_vector
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -293,8 +424,8 @@ int launch_fused_t(const WorldDev &w, const DT &tab, hipStream_t s) {
 }
 
 template <class DT>
-int launch_dispatch_t(const WorldDev &w, const DT &tab, hipStream_t s) {
-  if (dispatch_is_fused(w)) return launch_fused_t(w, tab, s);
+int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
+  if (dispatch_is_fused(w)) return launch_fused_t(w, tab, pick_vector, s);
   RouteSpan span{};
   span.v_begin = 0;
   span.v_count = w.G * w.M;
@@ -323,7 +454,7 @@ bool dispatch_is_fused(const WorldDev &w) {
   const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
   const bool exact = (w.Hb / 16) % kWave == 0;
   const bool row_fits = per_lane <= 8 || (exact && (per_lane == 14 || per_lane == 16));
-  return pairs <= kFusedMaxPairs && row_fits && 16 * w.K * 24 + (w.E + w.G) * 4 <= 48 * 1024;
+  return pairs <= kFusedMaxPairs && row_fits && fused_lds_bytes(w, 16, true) <= 60 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {
@@ -338,9 +469,10 @@ int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stre
   return (int)hipGetLastError();
 }
 
-int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, void *stream) {
-  if (inline_rows) return launch_dispatch_t(w, make_inline(w, inline_rows), (hipStream_t)stream);
-  return launch_dispatch_t(w, HbmDispatch{w.drank}, (hipStream_t)stream);
+int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t pick_vector, void *stream) {
+  if (pick_vector != 4 && pick_vector != 2) pick_vector = 1;
+  if (inline_rows) return launch_dispatch_t(w, make_inline(w, inline_rows), pick_vector, (hipStream_t)stream);
+  return launch_dispatch_t(w, HbmDispatch{w.drank}, pick_vector, (hipStream_t)stream);
 }
 
 }  // namespace pplx_amd

@@ -23,7 +23,8 @@ template <int NV, bool EXACT>
 __device__ __forceinline__ void load_row(const WorldDev &w, const DispatchRank &src, uint32_t t,
                                          uint32_t lane, RowRegs<NV> &regs) {
   const uint32_t nvec = w.Hb / 16;
-  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
+  const PPLX_GLOBAL u32x4 *row =
+      as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     uint32_t j = lane + i * kWave;
@@ -33,7 +34,7 @@ __device__ __forceinline__ void load_row(const WorldDev &w, const DispatchRank &
   regs.sc = 0.f;
   if (w.S) {
     const uint32_t j = lane < w.S ? lane : w.S - 1;
-    regs.sc = src.dp_xs[(int64_t)t * src.dp_xs_stride_row + (int64_t)j * src.dp_xs_stride_elem];
+    regs.sc = as_global(src.dp_xs)[(int64_t)t * src.dp_xs_stride_row + (int64_t)j * src.dp_xs_stride_elem];
   }
 }
 
@@ -94,7 +95,7 @@ __device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank 
       const int64_t step = (int64_t)read_lane64((uint64_t)dst.scale_step, k);
       if (lane < S) __builtin_nontemporal_store(regs.sc, sout + (int64_t)lane * step);
       if (S > kWave) {
-        const float *srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
+        const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
         for (uint32_t j = lane + kWave; j < S; j += kWave) {
           sout[(int64_t)j * step] = srow[(int64_t)j * src.dp_xs_stride_elem];
         }
