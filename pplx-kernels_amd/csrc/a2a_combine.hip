@@ -57,12 +57,14 @@ template <> struct Row8<_Float16> {
 template <typename U> struct Store8;
 template <> struct Store8<__bf16> {
   static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
-    __builtin_nontemporal_store(__builtin_convertvector(acc, bf16x8), reinterpret_cast<bf16x8 *>(row) + vec);
+    __builtin_nontemporal_store(__builtin_convertvector(acc, bf16x8),
+                                as_global(reinterpret_cast<bf16x8 *>(row)) + vec);
   }
 };
 template <> struct Store8<_Float16> {
   static __device__ __forceinline__ void at(void *row, uint32_t vec, const f32x8 &acc) {
-    __builtin_nontemporal_store(__builtin_convertvector(acc, f16x8), reinterpret_cast<f16x8 *>(row) + vec);
+    __builtin_nontemporal_store(__builtin_convertvector(acc, f16x8),
+                                as_global(reinterpret_cast<f16x8 *>(row)) + vec);
   }
 };
 
@@ -106,9 +108,9 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
   uint64_t row = 0;
   float weight = 0.f;
   if (lane < w.K) {
-    const uint32_t e = c.indices[(size_t)t * w.K + lane];
-    const uint32_t slot = w.slot_map[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
-    weight = c.weights[(int64_t)t * c.w_stride_row + lane];
+    const uint32_t e = as_global(c.indices)[(size_t)t * w.K + lane];
+    const uint32_t slot = as_global(w.slot_map)[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
+    weight = as_global(c.weights)[(int64_t)t * c.w_stride_row + lane];
     if (CT::kStaged) {
       // combine SEND left the row of (token, pick) in the staging area.
       if (e < w.E && slot != kInvalidSlot) {

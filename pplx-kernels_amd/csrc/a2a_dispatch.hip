@@ -61,7 +61,8 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   load_row<NV, EXACT>(w, src, t, lane, regs);
   Destination dst;
   if (lane < w.K) {
-    dst = resolve_destination(w, tab, src.indices[(size_t)t * w.K + lane], w.slot_map[(size_t)v * w.K + lane],
+    dst = resolve_destination(w, tab, as_global(src.indices)[(size_t)t * w.K + lane],
+                              as_global(w.slot_map)[(size_t)v * w.K + lane],
                               part == 0);
   }
   const uint32_t k0 = part * kper;
@@ -327,8 +328,8 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab)
   if (threadIdx.x < w.K) {
     uint64_t dst_row = 0, dst_scale = 0;
     int64_t step = 0;
-    const uint32_t e = src.indices[(size_t)t * w.K + threadIdx.x];
-    const uint32_t slot = w.slot_map[(size_t)v * w.K + threadIdx.x];
+    const uint32_t e = as_global(src.indices)[(size_t)t * w.K + threadIdx.x];
+    const uint32_t slot = as_global(w.slot_map)[(size_t)v * w.K + threadIdx.x];
     if (e < w.E && slot != kInvalidSlot) {
       const DispatchRank &dst = tab.at(e / w.L);
       const uint32_t el = e % w.L;
@@ -350,19 +351,20 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab)
   }
   __syncthreads();
   const uint32_t nvec = w.Hb / 16;
-  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
+  const PPLX_GLOBAL u32x4 *row =
+      as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
   for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) {
     const u32x4 x = row[j];
     for (uint32_t k = 0; k < w.K; ++k) {
-      if (s_row[k]) reinterpret_cast<u32x4 *>(s_row[k])[j] = x;
+      if (s_row[k]) global_ptr<u32x4>(s_row[k])[j] = x;
     }
   }
   if (w.S) {
-    const float *srow = src.dp_xs + (int64_t)t * src.dp_xs_stride_row;
+    const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
     for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) {
       const float sc = srow[(int64_t)j * src.dp_xs_stride_elem];
       for (uint32_t k = 0; k < w.K; ++k) {
-        if (s_scale[k]) reinterpret_cast<float *>(s_scale[k])[(int64_t)j * s_step[k]] = sc;
+        if (s_scale[k]) global_ptr<float>(s_scale[k])[(int64_t)j * s_step[k]] = sc;
       }
     }
   }

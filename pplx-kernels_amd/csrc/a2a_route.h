@@ -25,7 +25,7 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpa
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
   if (i < span.v_count && g < w.G && t < dispatch_group_tokens(w, tab, g)) {
-    const uint32_t *idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
+    const PPLX_GLOBAL uint32_t *idx = as_global(tab.at(g * w.dp + t % w.dp).indices) + (size_t)t * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
       if (e < w.E) atomicAdd(&lds_hist[e], 1u);
@@ -78,10 +78,10 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
   const bool in_span = i < span.v_count && g < w.G;
   const uint32_t n_group = in_span ? dispatch_group_tokens(w, tab, g) : 0;
   const bool live = in_span && t < n_group;
-  const uint32_t *idx = nullptr;
+  const PPLX_GLOBAL uint32_t *idx = nullptr;
   bool bad_expert = false;
   if (live) {
-    idx = tab.at(g * w.dp + t % w.dp).indices + (size_t)t * w.K;
+    idx = as_global(tab.at(g * w.dp + t % w.dp).indices) + (size_t)t * w.K;
     for (uint32_t k = 0; k < w.K; ++k) {
       const uint32_t e = idx[k];
       if (e < w.E) {
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
         // out_expert_num_tokens of the owning rank
         // (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).
         const DispatchRank &owner = tab.at(e / w.L);
-        owner.out_num_tokens[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
+        as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
       }
     }
   }
