@@ -418,6 +418,38 @@ def test_geometries(E, K, M, R):
     run_and_check(spec, generate(spec), use_numpy=True)
 
 
+@pytest.mark.parametrize("K,M", [(3, 40), (6, 40), (12, 40), (20, 30), (2, 700)])
+def test_one_launch_dispatch_pick_layouts(K, M):
+    """Small steps dispatch in one launch that reads the picks as vectors of 4, 2 or 1 ids: odd
+    and even K, K that leaves a last vector on its own, and more tokens than the workgroup has
+    threads (several passes over the earlier tokens)."""
+    spec = _small_spec(name=f"picks{K}", num_experts=64, experts_per_token=K, max_num_tokens=M, hidden_dim=128)
+    run_and_check(spec, generate(spec), use_numpy=True)
+
+
+@pytest.mark.parametrize("offset", [1, 2])
+def test_indices_at_odd_addresses(offset):
+    """indices only has to be contiguous (csrc/bindings/all_to_all_ops.cpp:150-153): a view that
+    starts 4 or 8 bytes into its storage must route like an aligned one."""
+    spec = _small_spec(name=f"odd{offset}", in_dtype=FP8, hidden_dim=512, num_experts=32, experts_per_token=8)
+    step = DeviceStep(spec, generate(spec))
+    for r, idx in enumerate(step.indices):
+        m, k = idx.shape
+        storage = torch.zeros(m * k + offset, dtype=torch.uint32, device="cuda")
+        view = storage[offset:].view(m, k)
+        view.copy_(idx)
+        assert view.data_ptr() % 16 == 4 * offset and view.is_contiguous()
+        step.indices[r] = view
+    world = make_world(spec, group_name=f"t-odd{offset}")
+    step.dispatch_world(world)
+    expected = check_dispatch_against_oracle(step)
+    step.expert_y_all.normal_()
+    step.combine_world(world)
+    assert world.faults() == 0
+    world.destroy()
+    check_combine_against_oracle(step, expected.slot_map)
+
+
 @pytest.mark.parametrize("api", ["world", "per_rank"])
 def test_more_ranks_than_inline_tables_hold(api):
     """Worlds beyond 64 ranks keep their rank tables in HBM, written by bind kernels."""
