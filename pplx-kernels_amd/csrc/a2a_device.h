@@ -118,8 +118,9 @@ struct SplitDev {
 // arguments each.
 constexpr uint32_t kInlineRanks = 64;
 constexpr uint32_t kBindBatch = 64;
-// Steps with at most this many (token, pick) pairs dispatch in one fused launch.
-constexpr uint32_t kFusedMaxPairs = 16384;
+// Steps of at most this many virtual tokens (DP groups x max_num_tokens) dispatch in one fused
+// launch.
+constexpr uint32_t kFusedMaxTokens = 16384;
 
 struct BindDispatchBatch {
   uint32_t first, count;

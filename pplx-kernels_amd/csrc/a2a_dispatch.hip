@@ -450,13 +450,15 @@ uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
 }
 
 bool dispatch_is_fused(const WorldDev &w) {
-  // Every workgroup recounts all earlier picks, so the one-launch form only pays
-  // while the whole step's routing is a few tens of KiB.
-  const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
+  // Every workgroup recounts all earlier tokens (work that grows with the square of the token
+  // count and sits on the ALU), so the one-launch form pays while that stays hidden behind the
+  // row traffic: measured against the three-launch form at 7 KiB rows it wins by 8 % (K = 8)
+  // and 4 % (K = 2) at 16384 tokens and loses from 32768 on.
+  const uint64_t tokens = (uint64_t)w.G * w.M;
   const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
   const bool exact = (w.Hb / 16) % kWave == 0;
   const bool row_fits = per_lane <= 8 || (exact && (per_lane == 14 || per_lane == 16));
-  return pairs <= kFusedMaxPairs && row_fits && fused_lds_bytes(w, 16, true) <= 60 * 1024;
+  return tokens <= kFusedMaxTokens && row_fits && fused_lds_bytes(w, 16, true) <= 60 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {

@@ -284,7 +284,8 @@ int main() {
       {"reference test, bf16 rows", 4, 2, 8, 3, 16, 10, 5, 2, 8, false},
       {"DSv3 row, 8 ranks x 16 tokens", 8, 1, 256, 8, 7168, 16, 1, 1, 56, true},
       {"72 ranks (tables in HBM)", 72, 1, 72, 2, 64, 3, 1, 2, 0, true},
-      {"1300 tokens (several routing tiles)", 2, 1, 8, 2, 64, 1300, 900, 2, 0, true},
+      {"1300 tokens (one launch, several counting passes)", 2, 1, 8, 2, 64, 1300, 900, 2, 0, true},
+      {"9000 tokens per rank (routing tiles + scatter)", 2, 1, 8, 2, 64, 9000, 7000, 2, 0, true},
   };
   bool ok = true;
   printf("libpplx_kernels %s\n", pplx_a2a_version());

@@ -18,7 +18,7 @@ def test_cpp_harness_passes():
     print(proc.stdout[-4000:], proc.stderr[-4000:])
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert "ALL PASSED" in proc.stdout
-    assert proc.stdout.count("  pass [") == 15
+    assert proc.stdout.count("  pass [") == 18
 
 
 def test_cpp_harness_is_built_and_linked_against_the_library():
