@@ -184,6 +184,7 @@ class _World:
         self.cfg = cfg_tuple
         self.ptr = ptr
         self.handles: set[int] = set()
+        self.experts_per_token = cfg_tuple[2]
         self.world_size = cfg_tuple[3]
         # A step's kernels are enqueued by the last rank to call, so the tensors of the
         # ranks that called earlier are kept alive until then: a temporary such as
@@ -362,9 +363,13 @@ def _check(cond: bool, msg: str) -> None:
 
 
 def _check_tensor(ndim: int, x: torch.Tensor, name: str) -> None:
-    _check(x.is_cuda, f"Tensor {name} must be on GPU")
-    _check(x.is_contiguous(), f"Tensor {name} must be contiguous")
-    _check(x.dim() == ndim, f"Tensor {name} must be {ndim} dimensional")
+    # (messages are only formatted on failure: these run on every call of the hot path)
+    if not x.is_cuda:
+        raise RuntimeError(f"Tensor {name} must be on GPU")
+    if not x.is_contiguous():
+        raise RuntimeError(f"Tensor {name} must be contiguous")
+    if x.dim() != ndim:
+        raise RuntimeError(f"Tensor {name} must be {ndim} dimensional")
 
 
 def _check_bound_m(bound_m: torch.Tensor | None) -> None:
@@ -506,15 +511,19 @@ def _dispatch(
     do_recv: bool,
 ) -> None:
     lib = load_library()
-    k = lib.pplx_a2a_num_experts_per_token(fptr)
+    world = _handle_world.get(fptr)
+    if world is None:
+        raise RuntimeError("pplx_kernels: invalid state: the handle has been destroyed")
     args = pack_dispatch_args(
-        k, out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m
-    )
+        world.experts_per_token, out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x,
+        dp_x_scale, indices, bound_m,
+    )  # fmt: skip
     mode = split_mode(do_send, do_recv)
-    with torch.cuda.device(indices.device):
-        check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
+    # The library selects the world's device for the launch and restores the caller's; the
+    # stream is the current one of the tensors' device (csrc/bindings/all_to_all_ops.cpp:163,194).
+    check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
     if mode == SPLIT_NONE:
-        _handle_world[fptr].hold(
+        world.hold(
             "dispatch",
             (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
         )
@@ -531,12 +540,14 @@ def _combine(
     do_recv: bool,
 ) -> None:
     lib = load_library()
+    world = _handle_world.get(fptr)
+    if world is None:
+        raise RuntimeError("pplx_kernels: invalid state: the handle has been destroyed")
     args = pack_combine_args(out_tokens, indices, weights, expert_y, bound_m)
     mode = split_mode(do_send, do_recv)
-    with torch.cuda.device(indices.device):
-        check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
+    check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
     if mode == SPLIT_NONE:
-        _handle_world[fptr].hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
+        world.hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
 
 
 def _fake_dispatch(*args, **kwargs) -> None:
