@@ -121,6 +121,9 @@ constexpr uint32_t kBindBatch = 64;
 // Steps of at most this many virtual tokens (DP groups x max_num_tokens) dispatch in one fused
 // launch.
 constexpr uint32_t kFusedMaxTokens = 16384;
+// A fused launch whose rows (all picks of all tokens) stay within this many bytes stores them
+// write-through into the 256 MB last-level cache instead of streaming them past it.
+constexpr uint64_t kWriteThroughMaxBytes = 128ull << 20;
 
 struct BindDispatchBatch {
   uint32_t first, count;

@@ -188,7 +188,7 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
 //      out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper,
-                                                              uint32_t pick_vector) {
+                                                              uint32_t pick_vector, uint32_t write_through) {
   extern __shared__ unsigned long long lds_u64[];
   constexpr bool kStaged = DT::kInline;
   constexpr uint32_t kTableWords = kStaged ? sizeof(DT) / 8 : 0;
@@ -310,7 +310,11 @@ __global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT t
   }
   const uint32_t k0 = my_part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  store_row<NV, EXACT>(w, my_src, my_t, lane, dst, k0, k1, regs);
+  if (write_through) {
+    store_row<NV, EXACT, true>(w, my_src, my_t, lane, dst, k0, k1, regs);
+  } else {
+    store_row<NV, EXACT, false>(w, my_src, my_t, lane, dst, k0, k1, regs);
+  }
 }
 
 // Rows longer than the register variants cover: stream each vector K times.
@@ -417,7 +421,10 @@ int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipSt
   const uint32_t tokens_per_block = kWaves / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
   const uint32_t lds = fused_lds_bytes(w, tokens_per_block, DT::kInline);
-#define PPLX_ROW_KERNEL_ARGS ksplit, kper, pick_vector
+  // Rows that fit the last-level cache with room to spare are written through into it.
+  const uint64_t row_bytes = (uint64_t)tokens * w.K * (w.Hb + 4ull * w.S);
+  const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper, pick_vector, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
