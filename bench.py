@@ -189,6 +189,27 @@ def cpu_baseline(spec, groups, budget_s=20.0):
     }
 
 
+def cpu_literal_loops(spec):
+    """One step in the literal per-token loops of the reference's test
+    (tests/test_all_to_all.py:113-120, 281-285), single core; only sensible for the smallest
+    workload (the loops are O(pairs) interpreter iterations)."""
+    import numpy as np
+
+    from oracle import a2a_oracle as orc
+    from tests.all_to_all_utils import ORACLE_DTYPE, generate, to_oracle_groups
+
+    og = to_oracle_groups(generate(spec))
+    M, E, K, H = spec.max_num_tokens, spec.num_experts, spec.experts_per_token, spec.hidden_dim
+    cap = M * spec.num_dp_groups
+    rng = np.random.default_rng(1)
+    expert_y = orc.from_float32(rng.standard_normal((E, cap, H), dtype=np.float32), ORACLE_DTYPE[spec.expert_y_dtype])
+    t0 = time.perf_counter()
+    res = orc.loop_dispatch(og, M, E, K, cap)
+    orc.loop_combine(og, M, E, K, H, expert_y, ORACLE_DTYPE[spec.expert_y_dtype], ORACLE_DTYPE[spec.out_dtype], res.slot_map)
+    return {"value": (time.perf_counter() - t0) * 1e6, "unit": "us", "cores": 1, "kind": "port",
+            "sample": "one full step, python loops over tokens and picks (oracle.a2a_oracle.loop_*)"}  # fmt: skip
+
+
 def counter_probe(spec, launches=3):
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a few eager dispatch and
     combine launches of the workload plus a plain elementwise copy of known size (1 GiB read,
@@ -326,6 +347,8 @@ def main() -> None:
             others[name], _, st = measure_workload(name, sp, k, min(args.warmup, 5))
             del st
             torch.cuda.empty_cache()
+            if name == "C1" and not args.no_cpu:
+                others[name]["cpu_literal_loops"] = cpu_literal_loops(sp)
         result["other_workloads"] = others
     print(json.dumps(result))
 
