@@ -272,14 +272,19 @@ __global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT t
   const bool pick_live = pick_exists && pick_t < ntok[pick_g];
   const uint32_t pick_e = pick_exists ? own_e[threadIdx.x] : w.E;
   uint32_t pick_slot = kInvalidSlot;
-  // (when all pick threads sit in one wave its LDS accesses are ordered by themselves)
+  // (when all pick threads sit in one wave the hardware keeps its LDS accesses in order by
+  // itself; the fence keeps the compiler from moving them across the rounds)
   const bool one_wave = own_pairs <= kWave;
   for (uint32_t j = 0; j < tokens_per_block; ++j) {
     if (pick_live && pick_j == j && pick_e < w.E) {
       pick_slot = hist[pick_e];
       hist[pick_e] = pick_slot + 1;
     }
-    if (!one_wave) __syncthreads();
+    if (one_wave) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    } else {
+      __syncthreads();
+    }
   }
   if (threadIdx.x < own_pairs) {
     Destination d;
