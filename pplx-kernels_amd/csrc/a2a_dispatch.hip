@@ -70,9 +70,11 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   store_row<NV, EXACT>(w, src, t, lane, dst, k0, k1, regs);
 }
 
-// dispatch_fused always runs with this many threads (16 waves): fewer, larger workgroups
-// repeat less counting, and a compile-time size keeps its first loads free of any wait.
-constexpr uint32_t kFusedThreads = 1024;
+// Threads of a dispatch_fused workgroup: 16 waves (fewer, larger workgroups repeat less
+// counting) while the row fits 8 registers of 16 bytes per lane, 8 waves for the 14- and
+// 16-register rows, which would spill under the 128-register limit of a 1024-thread workgroup.
+// A compile-time size also keeps the kernel's first loads free of any wait.
+constexpr uint32_t fused_threads(int nv) { return nv > 8 ? 512u : 1024u; }
 
 // A rank table that dispatch_fused has copied into LDS.
 struct LdsDispatch {
@@ -107,7 +109,7 @@ template <> struct PickVector<4> {
 // issued and before they are used: whatever it loads is in flight behind them (a wave's loads
 // complete in order).  The bookkeeping per token is one division: this loop is bound by the
 // ALU, not by memory, when every workgroup of a launch repeats it.
-template <int PV, class Table, class Between>
+template <int PV, uint32_t THREADS, class Table, class Between>
 __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows, uint32_t v_own,
                                            uint32_t v_own_end, uint32_t *hist, uint32_t *own_e,
                                            Between &&between) {
@@ -169,7 +171,7 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
   const Fetch first = issue(threadIdx.x);
   between();
   consume(threadIdx.x, first);
-  for (uint32_t v = threadIdx.x + kFusedThreads; v < v_own_end; v += kFusedThreads) consume(v, issue(v));
+  for (uint32_t v = threadIdx.x + THREADS; v < v_own_end; v += THREADS) consume(v, issue(v));
 }
 
 // Small steps: one launch does routing and scatter.  A workgroup owns tokens_per_block
@@ -187,8 +189,10 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
 //   4. the waves fan their rows out.  The last workgroup has counted everything and writes
 //      out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper,
-                                                              uint32_t pick_vector, uint32_t write_through) {
+__global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit,
+                                                                  uint32_t kper, uint32_t pick_vector,
+                                                                  uint32_t write_through) {
+  constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
   constexpr bool kStaged = DT::kInline;
   constexpr uint32_t kTableWords = kStaged ? sizeof(DT) / 8 : 0;
@@ -251,11 +255,11 @@ __global__ __launch_bounds__(kFusedThreads) void dispatch_fused(WorldDev w, DT t
     if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
   };
   if (pick_vector == 4) {
-    read_picks<4>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    read_picks<4, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
   } else if (pick_vector == 2) {
-    read_picks<2>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    read_picks<2, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
   } else {
-    read_picks<1>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    read_picks<1, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
   }
   if (counts_group) {
     uint32_t n = counted_bound ? counted_loaded : counted.m;
@@ -420,7 +424,7 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
 template <class DT>
 int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
-  constexpr uint32_t kWaves = kFusedThreads / kWave;
+  const uint32_t kWaves = fused_threads((int)((w.Hb / 16 + kWave - 1) / kWave)) / kWave;
   const uint32_t ksplit = pick_ksplit(w, kWaves);
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
   const uint32_t tokens_per_block = kWaves / ksplit;

@@ -145,3 +145,54 @@ def test_meta_kernels_are_no_ops():
     torch.ops.pplx_kernels.all_to_all_intranode_combine(
         0, m(4, 64), m(4, 2, dt=torch.uint32), m(4, 2, dt=torch.float32), m(2, 8, 64), None, True, True
     )
+
+
+def _gpu_kernels_of(path: str) -> list[dict]:
+    """Kernel metadata (AMDGPU code-object notes, msgpack) of every gfx code object embedded in
+    a host shared library."""
+    import struct
+
+    import msgpack
+
+    data = open(path, "rb").read()
+    kernels: list[dict] = []
+    pos = data.find(b"\x7fELF")
+    while pos >= 0:
+        if data[pos + 4] == 2 and struct.unpack_from("<H", data, pos + 18)[0] == 224:  # ELF64, EM_AMDGPU
+            (e_shoff,) = struct.unpack_from("<Q", data, pos + 0x28)
+            e_shentsize, e_shnum = struct.unpack_from("<HH", data, pos + 0x3A)
+            for i in range(e_shnum):
+                sh = pos + e_shoff + i * e_shentsize
+                (sh_type,) = struct.unpack_from("<I", data, sh + 4)
+                sh_offset, sh_size = struct.unpack_from("<QQ", data, sh + 0x18)
+                if sh_type != 7:  # SHT_NOTE
+                    continue
+                p, end = pos + sh_offset, pos + sh_offset + sh_size
+                while p < end:
+                    namesz, descsz, ntype = struct.unpack_from("<III", data, p)
+                    p += 12
+                    name = data[p : p + namesz]
+                    p += (namesz + 3) & ~3
+                    desc = data[p : p + descsz]
+                    p += (descsz + 3) & ~3
+                    if ntype == 32 and name.startswith(b"AMDGPU"):  # NT_AMDGPU_METADATA
+                        meta = msgpack.unpackb(desc, raw=False, strict_map_key=False)
+                        kernels += meta.get("amdhsa.kernels", [])
+        pos = data.find(b"\x7fELF", pos + 4)
+    return kernels
+
+
+def test_no_kernel_spills_or_uses_scratch():
+    """A kernel that spills registers needs scratch memory: its launch is several microseconds
+    slower and its spill traffic competes with the rows.  Every kernel of the library has to fit
+    its registers (this caught the 14- and 16-register row variants of the one-launch dispatch
+    under a 1024-thread workgroup)."""
+    kernels = _gpu_kernels_of(ops._LIB_PATH)
+    assert len(kernels) > 100
+    assert {k[".name"].split("ILi")[0] for k in kernels}  # names parsed
+    offenders = [
+        (k[".name"], k[".private_segment_fixed_size"], k.get(".vgpr_spill_count", 0), k.get(".sgpr_spill_count", 0))
+        for k in kernels
+        if k[".private_segment_fixed_size"] or k.get(".vgpr_spill_count", 0) or k.get(".sgpr_spill_count", 0)
+    ]
+    assert not offenders, offenders
