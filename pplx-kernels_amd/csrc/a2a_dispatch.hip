@@ -471,10 +471,7 @@ bool dispatch_is_fused(const WorldDev &w) {
   // row traffic: measured against the three-launch form at 7 KiB rows it wins by 8 % (K = 8)
   // and 4 % (K = 2) at 16384 tokens and loses from 32768 on.
   const uint64_t tokens = (uint64_t)w.G * w.M;
-  const uint32_t per_lane = (w.Hb / 16 + kWave - 1) / kWave;
-  const bool exact = (w.Hb / 16) % kWave == 0;
-  const bool row_fits = per_lane <= 8 || (exact && (per_lane == 14 || per_lane == 16));
-  return tokens <= kFusedMaxTokens && row_fits && fused_lds_bytes(w, 16, true) <= 60 * 1024;
+  return tokens <= kFusedMaxTokens && row_has_register_variant(w) && fused_lds_bytes(w, 16, true) <= 60 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {

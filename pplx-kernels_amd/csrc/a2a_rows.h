@@ -107,6 +107,20 @@ __device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank 
 }  // namespace
 }  // namespace pplx_amd
 
+namespace pplx_amd {
+namespace {
+// Rows of up to 8 KiB and rows of exactly 10, 12, 14 or 16 KiB (5120-, 6144-, 7168- and 8192-wide
+// bf16) have a register variant in every row kernel; other sizes beyond 8 KiB take
+// dispatch_scatter's padded variants or the streaming kernels.
+inline bool row_has_register_variant(const WorldDev &w) {
+  const uint32_t nvec = w.Hb / 16;
+  const uint32_t per_lane = (nvec + kWave - 1) / kWave;
+  const bool exact = nvec % kWave == 0;
+  return per_lane <= 8 || (exact && (per_lane == 10 || per_lane == 12 || per_lane == 14 || per_lane == 16));
+}
+}  // namespace
+}  // namespace pplx_amd
+
 // Picks the register variant for the row size and launches KERNEL<NV, EXACT, DT>.
 // Rows beyond 8 KiB exist only for dispatch_scatter (PPLX_LAUNCH_LARGE_ROW_VARIANT).
 #define PPLX_LAUNCH_ROW_VARIANT(KERNEL, NV, EXACT)                                               \
@@ -125,6 +139,8 @@ __device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank 
     else if (exact && per_lane == 6) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 6, true);                   \
     else if (exact && per_lane == 7) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 7, true);                   \
     else if (exact && per_lane == 8) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 8, true);                   \
+    else if (exact && per_lane == 10) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 10, true);                 \
+    else if (exact && per_lane == 12) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 12, true);                 \
     else if (exact && per_lane == 14) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 14, true);                 \
     else if (exact && per_lane == 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, true);                 \
     else if (per_lane <= 1) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 1, false);                           \

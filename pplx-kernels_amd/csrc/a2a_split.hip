@@ -232,9 +232,7 @@ int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const Disp
   int err = launch_route_t<DT, true>(w, tab, span, s);
   if (err) return err;
   const uint32_t lds = 0;
-  const uint32_t per_lane_rows = (w.Hb / 16 + kWave - 1) / kWave;
-  const bool exact_rows = (w.Hb / 16) % kWave == 0;
-  if (per_lane_rows > 8 && !(exact_rows && (per_lane_rows == 14 || per_lane_rows == 16))) {
+  if (!row_has_register_variant(w)) {
     hipLaunchKernelGGL(split_pack_long<DT>, dim3(w.M), dim3(256), 0, s, w, tab, g, member, sp);
     return (int)hipGetLastError();
   }
@@ -269,9 +267,7 @@ int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const Disp
   if (spread > 256) spread = 256;
   if (spread < 1) spread = 1;
   const dim3 grid(w.L * w.G, spread), block(256);
-  const uint32_t per_lane_rows = (w.Hb / 16 + kWave - 1) / kWave;
-  const bool exact_rows = (w.Hb / 16) % kWave == 0;
-  if (per_lane_rows > 8 && !(exact_rows && (per_lane_rows == 14 || per_lane_rows == 16))) {
+  if (!row_has_register_variant(w)) {
     hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, rank, sp);
     return (int)hipGetLastError();
   }

@@ -502,14 +502,18 @@ def test_hbm_tables_under_graph_replay():
     world.destroy()
 
 
-@pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 16384 + 32, 40960])
+@pytest.mark.parametrize(
+    "hidden_bytes", [16, 48, 1024 + 16, 4096, 7168, 8192, 10240, 12288, 14336, 16384, 16384 + 32, 40960]
+)
 def test_row_sizes(hidden_bytes):
-    """Rows from one 16-byte vector up to the streaming path for rows beyond 32 KiB."""
+    """Rows from one 16-byte vector up to the streaming path for rows beyond 32 KiB, with every
+    size that has an unpredicated register variant of its own (whole KiB up to 8, then 10, 12,
+    14 and 16 KiB)."""
     spec = _small_spec(name=f"row{hidden_bytes}", hidden_dim=hidden_bytes // 2, max_num_tokens=9)
     run_and_check(spec, generate(spec))
 
 
-@pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 16384 + 32])
+@pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 7168, 10240, 12288, 14336, 16384, 16384 + 32])
 def test_row_sizes_in_the_scatter_kernel(hidden_bytes):
     """The same row shapes where dispatch is routing tiles + scatter (> 16384 virtual tokens)."""
     spec = _small_spec(
@@ -619,6 +623,8 @@ def _combine_kw(step, r):
         dict(name="split-dp2", dp_size=2, in_dtype=FP8, hidden_dim=512),
         dict(name="split-tiles", max_num_tokens=1300, world_size=2, num_experts=8, hidden_dim=64),
         dict(name="split-longrow", hidden_dim=20480, max_num_tokens=6),
+        dict(name="split-10k-row", hidden_dim=5120, max_num_tokens=6),
+        dict(name="split-14k-row", hidden_dim=7168, max_num_tokens=6),
         dict(name="split-f32y", expert_y_dtype=torch.float32, out_dtype=torch.float16),
     ],
     ids=lambda kw: kw["name"],
