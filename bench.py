@@ -139,7 +139,14 @@ def measure_workload(name, spec, steps_k, warmup, detail=True):
                 both(steps[i % n_sets])()
             stream.synchronize()
             eager_us = (time.perf_counter() - t0) * 1e6 / min(steps_k, 50)
+        # the reference bench's one-way payload figures (tests/bench_all_to_all.py:131-139):
+        # pairs x bytes per dispatched token, pairs x bytes per combined row
+        pairs = out["pairs"]
+        disp_payload = pairs * (spec.hidden_dim_bytes + spec.hidden_dim_scale_bytes)
+        comb_payload = pairs * spec.hidden_dim * spec.out_dtype.itemsize
         out.update(
+            dispatch_payload_GBps=disp_payload / d_us / 1e3,
+            combine_payload_GBps=comb_payload / c_us / 1e3,
             dispatch_us=d_us,
             combine_us=c_us,
             dispatch_GBps=disp_b / d_us / 1e3,
