@@ -415,6 +415,8 @@ def test_combine_dtype_matrix(y_dtype, out_dtype):
         (512, 8, 300, 8), (1024, 4, 130, 4), (8, 8, 70, 2), (4, 1, 5, 1), (64, 6, 1500, 2), (2048, 2, 40, 2),
         # beyond 16384 virtual tokens the step takes the routing-tile kernels and the scatter
         (512, 8, 2100, 8), (2048, 2, 8300, 2), (64, 6, 4200, 4), (4, 1, 17000, 1), (1024, 3, 4200, 4),
+        # the limits of the build: 64 picks per token, 5440 experts (one 64-token chunk per routing tile)
+        (128, 64, 20, 4), (5440, 64, 3, 2),
     ],
 )  # fmt: skip
 def test_geometries(E, K, M, R):
@@ -422,6 +424,15 @@ def test_geometries(E, K, M, R):
     forms of dispatch (one launch up to 16384 virtual tokens, three beyond)."""
     spec = _small_spec(name=f"geo{E}", world_size=R, num_experts=E, experts_per_token=K, max_num_tokens=M, hidden_dim=128)
     run_and_check(spec, generate(spec), use_numpy=True)
+
+
+def test_most_experts_in_the_routing_tiles():
+    """5440 experts leave room for one 64-token chunk per routing tile: 282 tiles here."""
+    spec = _small_spec(name="e5440", num_experts=5440, experts_per_token=8, max_num_tokens=4500, hidden_dim=128)
+    groups = generate(spec)
+    for g in groups:
+        g.n = min(g.n, 150)
+    run_and_check(spec, groups, cap=max(int(expert_counts(groups, spec.num_experts).max()), 1), use_numpy=True)
 
 
 @pytest.mark.parametrize("K,M", [(3, 40), (6, 40), (12, 40), (20, 30), (2, 700)])
