@@ -78,7 +78,11 @@ class AllToAll:
         else:
             assert out_expert_x_scale is None
             assert dp_x_scale is None
-        self._dispatch_fn(
+        # Under torch.compile the call goes through the registered op (what the reference always
+        # does, src/pplx_kernels/all_to_all.py:47-59) so that it traces; an eager call skips the
+        # op dispatcher, which is a fifth of its host time, and runs the op's implementation.
+        fn = self._dispatch_fn if torch.compiler.is_compiling() else ops._dispatch
+        fn(
             self._ptr,
             out_expert_num_tokens,
             out_expert_x,
@@ -104,7 +108,8 @@ class AllToAll:
         """``out_tokens[t] = sum_k weights[t, k] * expert_y[slot of (t, k)]`` for
         ``t < bound_m``, fp32 accumulation in pick order; later rows are left as they are."""
         assert self._ptr is not None
-        self._combine_fn(
+        fn = self._combine_fn if torch.compiler.is_compiling() else ops._combine
+        fn(
             self._ptr,
             out_tokens,
             indices,
