@@ -605,8 +605,19 @@ int pplx_a2a_create(pplx_a2a_world_t *w, uint32_t rank, pplx_a2a_t **out) {
 int pplx_a2a_destroy(pplx_a2a_t *h) {
   if (!h) return PPLX_A2A_OK;
   {
-    std::lock_guard<std::mutex> lock(h->world->mu);
-    --h->world->attached;
+    pplx_a2a_world &w = *h->world;
+    std::lock_guard<std::mutex> lock(w.mu);
+    --w.attached;
+    // A rank that leaves in the middle of a step takes its half-made call with it, so that the
+    // handle which replaces it can call again.
+    if (w.arrived_dispatch[h->rank]) {
+      w.arrived_dispatch[h->rank] = 0;
+      --w.n_arrived_dispatch;
+    }
+    if (w.arrived_combine[h->rank]) {
+      w.arrived_combine[h->rank] = 0;
+      --w.n_arrived_combine;
+    }
   }
   delete h;
   return PPLX_A2A_OK;

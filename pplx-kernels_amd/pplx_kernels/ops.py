@@ -189,13 +189,18 @@ class _World:
         # A step's kernels are enqueued by the last rank to call, so the tensors of the
         # ranks that called earlier are kept alive until then: a temporary such as
         # ``x.to(device)`` must not go back to the caching allocator before it is read.
-        self.pending: dict[str, list] = {"dispatch": [], "combine": []}
+        self.pending: dict[str, dict[int, tuple]] = {"dispatch": {}, "combine": {}}
 
-    def hold(self, kind: str, tensors: tuple) -> None:
+    def hold(self, kind: str, fptr: int, tensors: tuple) -> None:
         held = self.pending[kind]
-        held.append(tensors)
+        held[fptr] = tensors
         if len(held) >= self.world_size:
             held.clear()
+
+    def release(self, fptr: int) -> None:
+        """A handle that is destroyed in the middle of a step takes its half-made calls along."""
+        for held in self.pending.values():
+            held.pop(fptr, None)
 
 
 _worlds: dict[str, _World] = {}
@@ -271,6 +276,7 @@ def _destroy(fptr: int) -> None:
             raise RuntimeError(f"pplx_kernels: unknown all-to-all handle {fptr:#x}")
         check_status(lib.pplx_a2a_destroy(fptr))
         world.handles.discard(fptr)
+        world.release(fptr)
         if not world.handles:
             check_status(lib.pplx_a2a_world_destroy(world.ptr))
             _worlds.pop(world.key, None)
@@ -525,6 +531,7 @@ def _dispatch(
     if mode == SPLIT_NONE:
         world.hold(
             "dispatch",
+            fptr,
             (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
         )
 
@@ -547,7 +554,7 @@ def _combine(
     mode = split_mode(do_send, do_recv)
     check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
     if mode == SPLIT_NONE:
-        world.hold("combine", (out_tokens, indices, weights, expert_y, bound_m))
+        world.hold("combine", fptr, (out_tokens, indices, weights, expert_y, bound_m))
 
 
 def _fake_dispatch(*args, **kwargs) -> None:

@@ -797,6 +797,31 @@ def test_torch_cuda_graph_with_per_rank_calls():
 # ---------------------------------------------------------------------------
 # Error behaviour
 # ---------------------------------------------------------------------------
+def test_a_rank_replaced_in_the_middle_of_a_step():
+    """A handle destroyed after its dispatch call, before the step is complete, takes that call
+    with it: the handle that replaces it calls again and the step comes out whole."""
+    spec = _small_spec(name="replace", in_dtype=FP8, hidden_dim=512)
+    step = DeviceStep(spec, generate(spec))
+    ranks = _make_ranks(spec, "replace")
+    ranks[0].dispatch(**_dispatch_kw(step, 0))
+    ranks[0].destroy()
+    from pplx_kernels import AllToAll
+
+    ranks[0] = AllToAll.intranode(
+        spec.max_num_tokens, spec.num_experts, spec.experts_per_token, 0, spec.world_size, spec.dp_size,
+        spec.hidden_dim, spec.hidden_dim_bytes, spec.hidden_dim_scale_bytes, group_name="replace",
+    )  # fmt: skip
+    for r in range(spec.world_size):
+        ranks[r].dispatch(**_dispatch_kw(step, r))
+    expected = check_dispatch_against_oracle(step)
+    step.expert_y_all.normal_()
+    for r in range(spec.world_size):
+        ranks[r].combine(**_combine_kw(step, r))
+    check_combine_against_oracle(step, expected.slot_map)
+    for a in ranks:
+        a.destroy()
+
+
 def test_errors_are_runtime_errors():
     from pplx_kernels import AllToAll
 
