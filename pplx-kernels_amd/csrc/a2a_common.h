@@ -60,22 +60,37 @@ __device__ __forceinline__ PPLX_GLOBAL V *as_global(V *p) {
   return (PPLX_GLOBAL V *)p;
 }
 
-// Row stores come in two cache policies.  Non-temporal: the data streams past the caches to
-// HBM, which suits a step that writes more than the 256 MB last-level cache holds.  Agent-scope
-// write-through ("sc1"): the data stays in the last-level cache, where the experts' GEMMs will
-// look for it next, and a step whose rows fit there no longer waits for HBM to take them
-// (dispatch of 8 x 128 DSv3 tokens: 18.9 instead of 22.6 us; from about 240 MB per step on it
-// is the slower of the two).  The compiler offers no builtin for the second, hence the asm; it
-// is a plain vector store.
-template <bool WRITE_THROUGH, typename V>
+// Cache policy of a row store.
+//   kStream        non-temporal: the data streams past the caches to HBM, which suits a step
+//                  that writes more than the 256 MB last-level cache holds;
+//   kStreamThrough non-temporal and written through at agent scope ("sc1 nt"): 1.5-2 % faster
+//                  than kStream in the scatter of steps of 32768 tokens and more, 1-2 % slower
+//                  in the one-launch dispatch of 8192-token steps;
+//   kKeep          written through at agent scope ("sc1"): the data stays in the last-level
+//                  cache, where the experts' GEMMs will look for it next, and a step whose rows
+//                  fit there no longer waits for HBM to take them (dispatch of 8 x 128 DSv3
+//                  tokens: 18.9 instead of 22.6 us; from about 240 MB per step on it is the
+//                  slowest of the three).
+// The compiler offers no builtin for the scoped forms, hence the asm; they are plain vector stores.
+enum class RowStore { kStream, kStreamThrough, kKeep };
+
+template <RowStore POLICY, typename V>
 __device__ __forceinline__ void row_store(V v, PPLX_GLOBAL V *p) {
-  if constexpr (!WRITE_THROUGH) {
+  static_assert(sizeof(V) == 16 || sizeof(V) == 4, "row_store: 4- or 16-byte values");
+  if constexpr (POLICY == RowStore::kStream) {
     __builtin_nontemporal_store(v, p);
-  } else if constexpr (sizeof(V) == 16) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+  } else if constexpr (POLICY == RowStore::kStreamThrough) {
+    if constexpr (sizeof(V) == 16) {
+      asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+    } else {
+      asm volatile("global_store_dword %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+    }
   } else {
-    static_assert(sizeof(V) == 4, "row_store: 4- or 16-byte values");
-    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    if constexpr (sizeof(V) == 16) {
+      asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    } else {
+      asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    }
   }
 }
 

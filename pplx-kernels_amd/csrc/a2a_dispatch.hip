@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   }
   const uint32_t k0 = part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  store_row<NV, EXACT>(w, src, t, lane, dst, k0, k1, regs);
+  store_row<NV, EXACT, RowStore::kStreamThrough>(w, src, t, lane, dst, k0, k1, regs);
 }
 
 // Threads of a dispatch_fused workgroup: 16 waves (fewer, larger workgroups repeat less
@@ -320,9 +320,9 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   const uint32_t k0 = my_part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
   if (write_through) {
-    store_row<NV, EXACT, true>(w, my_src, my_t, lane, dst, k0, k1, regs);
+    store_row<NV, EXACT, RowStore::kKeep>(w, my_src, my_t, lane, dst, k0, k1, regs);
   } else {
-    store_row<NV, EXACT, false>(w, my_src, my_t, lane, dst, k0, k1, regs);
+    store_row<NV, EXACT, RowStore::kStream>(w, my_src, my_t, lane, dst, k0, k1, regs);
   }
 }
 
