@@ -797,6 +797,47 @@ def test_torch_cuda_graph_with_per_rank_calls():
 # ---------------------------------------------------------------------------
 # Error behaviour
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_geometries(seed):
+    """Forty geometries per seed drawn at random (ranks, DP size, experts, top-k, tokens, row
+    width, dtypes, routing skew, ragged and empty ranks, both call forms), each against the
+    oracle: dispatch bit-exact, combine within tolerance."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(40):
+        dp = rng.choice([1, 1, 1, 2, 4])
+        groups_n = rng.choice([1, 2, 3, 4, 8, 16])
+        R = groups_n * dp
+        E = R * rng.choice([1, 2, 3, 8, 32])
+        K = rng.choice([k for k in [1, 2, 3, 4, 6, 7, 8, 12, 16] if k <= E])
+        big = rng.random() < 0.15 and groups_n <= 4
+        M = rng.choice([5000, 9000, 17000]) if big else rng.choice([1, 2, 5, 17, 64, 130, 700])
+        M = min(M, 40000 // groups_n)
+        fp8 = rng.random() < 0.5
+        if fp8:
+            H = 512 if big else rng.choice([512, 1024, 2048, 7168])
+        else:
+            H = rng.choice([8, 64]) if big else rng.choice([8, 24, 64, 520, 1024, 2880, 5120])
+        spec = WorkloadSpec(
+            f"rnd{seed}-{it}", 900 + it, R, E, K, H, M, FP8 if fp8 else rng.choice([torch.bfloat16, torch.float16]),
+            out_dtype=rng.choice([torch.bfloat16, torch.float16]),
+            expert_y_dtype=rng.choice([torch.float32, torch.bfloat16, torch.float16]),
+            dp_size=dp, tokens=rng.choice(["max", "uniform"]), routing=rng.choice(["uniform", "zipf:1.0", "mix:1.2"]),
+        )  # fmt: skip
+        groups = generate(spec)
+        for g in groups:
+            if big:
+                g.n = min(g.n, rng.choice([0, 50, 300]))
+            elif rng.random() < 0.05:
+                g.n = 0
+        cap = max(int(expert_counts(groups, E).max()), 1)
+        with_bound_m = rng.random() < 0.8 or any(g.n != M for g in groups)
+        run_and_check(
+            spec, groups, api=rng.choice(["world", "per_rank"]), cap=cap, with_bound_m=with_bound_m, use_numpy=True
+        )  # fmt: skip
+
+
 def test_a_rank_replaced_in_the_middle_of_a_step():
     """A handle destroyed after its dispatch call, before the step is complete, takes that call
     with it: the handle that replaces it calls again and the step comes out whole."""
