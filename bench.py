@@ -144,7 +144,25 @@ def measure_workload(name, spec, steps_k, warmup, detail=True):
         pairs = out["pairs"]
         disp_payload = pairs * (spec.hidden_dim_bytes + spec.hidden_dim_scale_bytes)
         comb_payload = pairs * spec.hidden_dim * spec.out_dtype.itemsize
+        # eager launches of steps packed once (LoopbackWorld.bind): two library calls per step,
+        # same rotating buffer sets, HIP events on the launch stream
+        bound = [st.bind_world(world) for st in steps]
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            for i in range(warmup):
+                bound[i % n_sets].dispatch(stream)
+                bound[i % n_sets].combine(stream)
+            stream.synchronize()
+            start.record(stream)
+            for i in order:
+                bound[i].dispatch(stream)
+                bound[i].combine(stream)
+            end.record(stream)
+            stream.synchronize()
+        bound_us = start.elapsed_time(end) * 1e3 / len(order)
+        del bound
         out.update(
+            bound_eager_step_us=bound_us,
             dispatch_payload_GBps=disp_payload / d_us / 1e3,
             combine_payload_GBps=comb_payload / c_us / 1e3,
             dispatch_us=d_us,
@@ -314,14 +332,24 @@ def main() -> None:
         "launches_timed": reps * n_sets * launches_per_graph,
     }
 
+    # A step can be launched two ways: replaying a captured hipGraph, or two eager library calls
+    # on arguments packed once (LoopbackWorld.bind).  Both run the same kernels on the same
+    # rotating buffer sets; the headline is the faster one and says which (on this stack one
+    # hipGraphLaunch call costs more host time than two eager launches).
+    graph_us, bound_us = main_res["step_us"], main_res["bound_eager_step_us"]
+    best_us = min(graph_us, bound_us)
+    timed = (
+        f"{'eager launches of a bound step (LoopbackWorld.bind)' if bound_us <= graph_us else 'hipGraph replay'}"
+        f" of dispatch+combine, rotating buffer sets; hipGraph replay {graph_us:.1f} us, bound eager {bound_us:.1f} us"
+    )
     result = {
         "metric": "dispatch+combine latency (us) and achieved HBM GB/s, DSv3 shape 128 tok/rank, 1 GPU",
-        "value": main_res["step_us"],
+        "value": best_us,
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": main_res["step_us"] / 1e3,
+        "ms_per_step": best_us / 1e3,
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
@@ -336,7 +364,7 @@ def main() -> None:
             "tokens_per_rank": spec.max_num_tokens,
             "in_dtype": str(spec.in_dtype).replace("torch.", ""),
             "out_dtype": str(spec.out_dtype).replace("torch.", ""),
-            "timed": "hipGraph replay of dispatch+combine, rotating buffer sets",
+            "timed": timed,
         },
         "roofline": roofline,
         "detail": main_res,

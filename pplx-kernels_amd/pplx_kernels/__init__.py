@@ -4,5 +4,6 @@ no SHMEM layer)."""
 
 from . import ops as ops
 from .all_to_all import AllToAll as AllToAll
+from .loopback import BoundStep as BoundStep
 from .loopback import Graph as Graph
 from .loopback import LoopbackWorld as LoopbackWorld

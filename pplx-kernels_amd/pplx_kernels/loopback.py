@@ -46,6 +46,35 @@ class Graph:
             pass
 
 
+class BoundStep:
+    """One step's arguments of all ranks, checked and packed once: ``dispatch()`` and
+    ``combine()`` then cost one library call each, with no per-rank work in Python.  The eager
+    alternative to :class:`Graph` for a caller whose buffers stay where they are from step to
+    step (on this stack a graph replay costs more host time than two eager launches).  The
+    tensors are kept alive by the object; their contents may change between calls, their
+    addresses, shapes and strides may not."""
+
+    def __init__(self, world: "LoopbackWorld", dispatch_args, combine_args, device, keep: tuple) -> None:
+        self._world = world
+        self._dispatch_args = dispatch_args
+        self._combine_args = combine_args
+        self._device = device
+        self._keep = keep
+        self._lib = ops.load_library()
+
+    def dispatch(self, stream: torch.cuda.Stream | None = None) -> None:
+        s = stream if stream is not None else torch.cuda.current_stream(self._device)
+        ops.check_status(
+            self._lib.pplx_a2a_world_dispatch(self._world._world_ptr, self._dispatch_args, s.cuda_stream)
+        )
+
+    def combine(self, stream: torch.cuda.Stream | None = None) -> None:
+        s = stream if stream is not None else torch.cuda.current_stream(self._device)
+        ops.check_status(
+            self._lib.pplx_a2a_world_combine(self._world._world_ptr, self._combine_args, s.cuda_stream)
+        )
+
+
 class LoopbackWorld:
     def __init__(
         self,
@@ -131,6 +160,36 @@ class LoopbackWorld:
         ops.check_status(
             ops.load_library().pplx_a2a_world_combine(self._world_ptr, self._combine_args, stream)
         )
+
+    def bind(
+        self,
+        out_expert_num_tokens: Sequence[torch.Tensor],
+        out_expert_x: Sequence[torch.Tensor],
+        out_expert_x_scale: Sequence[torch.Tensor | None],
+        dp_x: Sequence[torch.Tensor],
+        dp_x_scale: Sequence[torch.Tensor | None],
+        indices: Sequence[torch.Tensor],
+        bound_m: Sequence[torch.Tensor | None],
+        out_tokens: Sequence[torch.Tensor],
+        weights: Sequence[torch.Tensor],
+        expert_y: Sequence[torch.Tensor],
+    ) -> BoundStep:
+        """Checks and packs the arguments of :meth:`dispatch` and :meth:`combine` once and
+        returns a :class:`BoundStep` that launches them as often as wanted."""
+        d_args = (ops.DispatchArgs * self.world_size)()
+        c_args = (ops.CombineArgs * self.world_size)()
+        for r in range(self.world_size):
+            ops.pack_dispatch_args(
+                self.experts_per_token, out_expert_num_tokens[r], out_expert_x[r], out_expert_x_scale[r],
+                dp_x[r], dp_x_scale[r], indices[r], bound_m[r], out=d_args[r],
+            )  # fmt: skip
+            ops.pack_combine_args(out_tokens[r], indices[r], weights[r], expert_y[r], bound_m[r], out=c_args[r])
+        keep = tuple(
+            list(seq)
+            for seq in (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices,
+                        bound_m, out_tokens, weights, expert_y)
+        )  # fmt: skip
+        return BoundStep(self, d_args, c_args, indices[0].device, keep)
 
     def faults(self) -> int:
         """Sticky device-side fault bits since the last call (synchronises the stream):

@@ -285,6 +285,12 @@ class DeviceStep:
     def combine_world(self, world) -> None:
         world.combine(self.out_tokens, self.indices, self.weights, self.expert_y, self.bound_m)
 
+    def bind_world(self, world):
+        return world.bind(
+            self.expert_num_tokens, self.expert_x, self.expert_x_scale, self.dp_x, self.dp_x_scale,
+            self.indices, self.bound_m, self.out_tokens, self.weights, self.expert_y,
+        )  # fmt: skip
+
     def dispatch_per_rank(self, ranks) -> None:
         for r, ata in enumerate(ranks):
             ata.dispatch(

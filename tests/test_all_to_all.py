@@ -754,6 +754,34 @@ def test_graph_replay_decode_shape():
     world.destroy()
 
 
+def test_bound_step_relaunches_with_new_inputs():
+    """LoopbackWorld.bind packs a step once; every launch afterwards reads the tensors' current
+    contents (inputs, routing and bound_m change between launches here)."""
+    spec = baseline_configs()["C3"]
+    step = DeviceStep(spec, generate(spec))
+    world = make_world(spec, group_name="bound")
+    bound = step.bind_world(world)
+    step.expert_y_all.normal_()
+    for it in range(3):
+        new = generate(spec, seed=300 + it)
+        for r, g in enumerate(new):
+            if it == 1 and r % 5 == 0:
+                g.n = 0
+            step.dp_x[r].copy_(g.x.cuda())
+            step.dp_x_scale[r].copy_(g.x_scale.cuda())
+            step.indices[r].copy_(g.indices.cuda().to(torch.uint32))
+            step.weights[r].copy_(g.weights.cuda())
+            step.bound_m[r].copy_(torch.tensor([g.n], dtype=torch.uint32).cuda())
+            step.out_tokens[r].fill_(float("nan"))
+        step.groups = new
+        bound.dispatch()
+        bound.combine()
+        expected = check_dispatch_against_oracle(step)
+        check_combine_against_oracle(step, expected.slot_map)
+    assert world.faults() == 0
+    world.destroy()
+
+
 def test_torch_cuda_graph_with_per_rank_calls():
     """The reference's "CUDA graph support" as a torch user meets it: torch.cuda.graph around
     the per-rank AllToAll calls, replayed with new inputs and a new bound_m."""
