@@ -20,9 +20,13 @@
  *     thread's last failure.
  *   - Device pointers are HBM addresses on the world's device.  `stream` is a
  *     hipStream_t passed as void* (NULL = the legacy default stream).
- *   - No entry point other than *_create / *_destroy allocates, frees or
- *     synchronises; dispatch/combine only enqueue kernels, so they may be
- *     captured in a hipGraph and replayed.
+ *   - Only *_create, *_destroy and pplx_a2a_world_reserve_split allocate, free
+ *     or synchronise (pplx_a2a_world_faults synchronises the stream it reads
+ *     behind); dispatch / combine only enqueue kernels, so they may be captured
+ *     in a hipGraph and replayed.
+ *   - Outputs of a send+recv step made of per-rank calls are valid once the
+ *     LAST rank's call has returned, in stream order of any stream a rank of
+ *     the step called on.
  */
 #ifndef PPLX_A2A_H_
 #define PPLX_A2A_H_
@@ -101,7 +105,7 @@ typedef struct pplx_a2a_dispatch_args {
   const float *dp_x_scale;               /* [m, S] or NULL */
   int64_t dp_x_scale_stride_elem;        /* floats */
   int64_t dp_x_scale_stride_row;         /* floats */
-  const uint32_t *indices;               /* [m, K] contiguous, distinct experts per row */
+  const uint32_t *indices;               /* [m, K] contiguous */
   uint32_t m;                            /* rows of dp_x / indices */
   const uint32_t *bound_m;               /* device scalar: tokens actually present, or NULL (= m) */
 } pplx_a2a_dispatch_args_t;
@@ -146,10 +150,22 @@ uint32_t pplx_a2a_rank(const pplx_a2a_t *handle);
 
 /* AllToAllIntraNode::dispatch, csrc/all_to_all/intranode_dispatch.cu:288-390.
  * The call is collective over the world, like the reference's: with
- * PPLX_A2A_SPLIT_NONE the kernels are enqueued on `stream` when the last of
- * the world_size ranks has made its call for the step, and every rank's
- * outputs are complete once they finish.  With SEND / RECV, every rank's SEND
- * must be enqueued before the first RECV. */
+ * PPLX_A2A_SPLIT_NONE the kernels are enqueued when the last of the world_size
+ * ranks has made its call for the step, on that call's `stream`, and every
+ * rank's outputs are complete once they finish.  Ranks may call on different
+ * streams (csrc/bindings/all_to_all_ops.cpp:163,194 runs each rank on its own
+ * current stream): the launching stream first waits for the work the other
+ * streams held when the last call came in, and those streams then wait for the
+ * kernels; work a rank enqueues BETWEEN its own call and the last rank's call
+ * is not ordered against the step.  The ranks of a captured step must share
+ * one stream (PPLX_A2A_INVALID_STATE otherwise).
+ * With SEND / RECV a call enqueues at once on its `stream`: every rank's SEND
+ * must be enqueued before the first RECV, staging must have been reserved with
+ * pplx_a2a_world_reserve_split (PPLX_A2A_INVALID_STATE otherwise), and ranks on
+ * different streams order them themselves.
+ * Without bound_m, m may not exceed max_num_tokens
+ * (csrc/all_to_all/intranode_dispatch.cu:65); the members of a DP group must
+ * pass the same m. */
 int pplx_a2a_dispatch(pplx_a2a_t *handle, const pplx_a2a_dispatch_args_t *args,
                       int split_mode, void *stream);
 /* AllToAllIntraNode::combine<T,U>, csrc/all_to_all/intranode_combine.cu:190-266. */
@@ -166,10 +182,25 @@ int pplx_a2a_world_dispatch(pplx_a2a_world_t *world, const pplx_a2a_dispatch_arg
 int pplx_a2a_world_combine(pplx_a2a_world_t *world, const pplx_a2a_combine_args_t *per_rank,
                            void *stream);
 
+/* Allocates the staging that split send / recv calls go through (the reference
+ * allocates its inboxes in the constructor, csrc/all_to_all/intranode.cpp:37-136;
+ * here a world that never splits does not pay for them): about
+ * G*M*K * (hidden_dim_bytes + hidden_dim_scale_bytes + 16) bytes for dispatch plus
+ * G*M*K * hidden_dim * expert_y_elem_bytes for combine (0 = dispatch only, 2 =
+ * bf16 / f16 expert_y, 4 = also f32).  May be called again with a wider element
+ * while no split combine step is in flight.  Synchronises the device. */
+int pplx_a2a_world_reserve_split(pplx_a2a_world_t *world, uint32_t expert_y_elem_bytes);
+
 /* Reads and clears the world's device-side fault word (synchronises `stream`):
  * bit 0 = a routed row did not fit out_expert_x_rows and was dropped,
  * bit 1 = an expert index >= num_experts was ignored,
- * bit 2 = combine met a slot beyond expert_y_rows. */
+ * bit 2 = combine met a slot beyond expert_y_rows,
+ * bit 3 = an expert id repeated inside one token: the repeat took no row, was
+ *         not counted and adds nothing in combine (the reference gives every
+ *         pick a slot, csrc/all_to_all/intranode_dispatch.cu:139-144; top-k
+ *         routing never repeats an expert),
+ * bit 4 = a bound_m beyond max_num_tokens (or beyond m) was clamped
+ *         (csrc/all_to_all/intranode_dispatch.cu:65 asserts). */
 int pplx_a2a_world_faults(pplx_a2a_world_t *world, void *stream, uint32_t *out_bits);
 
 /* ---- hipGraph plumbing ------------------------------------------------ */
@@ -187,6 +218,8 @@ int pplx_a2a_graph_destroy(pplx_a2a_graph_t *graph);
 const char *pplx_a2a_last_error(void);
 /* "major.minor.patch" of this library. */
 const char *pplx_a2a_version(void);
+/* Hash of the sources the library was built from (a binding can tell a stale build). */
+const char *pplx_a2a_build_id(void);
 
 #ifdef __cplusplus
 }

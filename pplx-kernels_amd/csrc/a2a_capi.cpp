@@ -19,6 +19,13 @@
 #include "a2a_device.h"
 #include "pplx_a2a.h"
 
+// Profiler ranges around the launch sequences, like the reference's nvtxRangePush("dispatch") /
+// ("combine") (csrc/all_to_all/intranode_dispatch.cu:354,389, intranode_combine.cu:245,265).
+// The build links the roctx library when its header is installed.
+#ifdef PPLX_A2A_ROCTX
+#include <rocprofiler-sdk-roctx/roctx.h>
+#endif
+
 using namespace pplx_amd;
 
 namespace {
@@ -51,6 +58,24 @@ int fail(int status, const char *fmt, ...) {
   } while (0)
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+class ProfilerRange {
+ public:
+  explicit ProfilerRange(const char *name) {
+#ifdef PPLX_A2A_ROCTX
+    roctxRangePushA(name);
+#else
+    (void)name;
+#endif
+  }
+  ~ProfilerRange() {
+#ifdef PPLX_A2A_ROCTX
+    roctxRangePop();
+#endif
+  }
+  ProfilerRange(const ProfilerRange &) = delete;
+  ProfilerRange &operator=(const ProfilerRange &) = delete;
+};
 
 // Restores the caller's current device on scope exit.
 class DeviceScope {
@@ -96,11 +121,18 @@ struct pplx_a2a_world {
   // Capture session that recorded the last bind of each table (0 = an eager bind).
   unsigned long long bind_capture_dispatch = 0, bind_capture_combine = 0;
 
-  // Split send / recv mode: staging is allocated by the first split call; the masks record
-  // which ranks have made which call of the step in flight.
+  // Streams the ranks of the step being assembled called on (per-rank calls), and the events
+  // that order them against the stream of the last caller, which gets the kernels.
+  std::vector<void *> stream_dispatch, stream_combine;
+  std::vector<hipEvent_t> rank_events;  // [R]
+  hipEvent_t done_event = nullptr;
+
+  // Split send / recv mode: staging is allocated by pplx_a2a_world_reserve_split; the masks
+  // record which ranks have made which call of the step in flight.
   SplitDev split{};
   bool split_ready = false;
-  std::vector<uint8_t> dsend, drecv, csend, crecv;
+  uint32_t split_y_elem_bytes = 0;  // widest expert_y element the combine staging holds
+  std::vector<uint8_t> dsend, drecv, csend, crecv, group_routed;
   uint32_t n_dsend = 0, n_drecv = 0, n_csend = 0, n_crecv = 0;
   int split_in_dtype = -1;
 };
@@ -166,6 +198,10 @@ int convert_dispatch(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_disp
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: dp_x must be 16-byte aligned with a 16-byte row stride", rank);
   if (a.out_expert_x_rows < 0)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x_rows is negative", rank);
+  // csrc/all_to_all/intranode_dispatch.cu:65 asserts numSendTokens <= maxNumTokens; a device-side
+  // bound_m beyond the limit is clamped and reported through the fault word instead.
+  if (!a.bound_m && a.m > w.dev.M)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, w.dev.M);
   const uint64_t rows = a.out_expert_x_rows ? (uint64_t)a.out_expert_x_rows : (uint64_t)w.dev.M * w.dev.G;
   DispatchRank d{};
   d.out_num_tokens = a.out_expert_num_tokens;
@@ -212,6 +248,8 @@ int convert_combine(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_combi
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_tokens must be 16-byte aligned with a 16-byte row stride", rank);
   if (a.expert_y_rows < 0)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y_rows is negative", rank);
+  if (!a.bound_m && a.m > w.dev.M)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, w.dev.M);
   const uint64_t rows = a.expert_y_rows ? (uint64_t)a.expert_y_rows : (uint64_t)w.dev.M * w.dev.G;
   CombineRank c{};
   c.out_tokens = a.out_tokens;
@@ -275,23 +313,91 @@ int flush_table(pplx_a2a_world &w, const std::vector<Row> &rows, std::vector<Row
   return PPLX_A2A_OK;
 }
 
-// Widest load (in expert ids) that suits the indices of every rank of the pending step.
-uint32_t pick_vector_of(const pplx_a2a_world &w) {
-  uint32_t pv = w.dev.K % 4 == 0 ? 4 : w.dev.K % 2 == 0 ? 2 : 1;
-  for (const DispatchRank &r : w.pend_dispatch) {
-    const uintptr_t p = reinterpret_cast<uintptr_t>(r.indices);
-    while (pv > 1 && p % (4 * pv) != 0) pv /= 2;
-  }
+// Widest load (in expert ids) that suits a row of K picks starting at `indices`.
+uint32_t pick_vector_for(uint32_t K, const uint32_t *indices, uint32_t at_most = 4) {
+  uint32_t pv = K % 4 == 0 ? 4 : K % 2 == 0 ? 2 : 1;
+  if (pv > at_most) pv = at_most;
+  const uintptr_t p = reinterpret_cast<uintptr_t>(indices);
+  while (pv > 1 && p % (4 * pv) != 0) pv /= 2;
   return pv;
 }
 
+// ... that suits the indices of every rank of the pending step.
+uint32_t pick_vector_of(const pplx_a2a_world &w) {
+  uint32_t pv = 4;
+  for (const DispatchRank &r : w.pend_dispatch) pv = pick_vector_for(w.dev.K, r.indices, pv);
+  return pv;
+}
+
+// The members of a DP group hold the same tokens (csrc/all_to_all/intranode_dispatch.cu:97
+// strides one token list over them), so they must agree on how many rows there are: the
+// kernels take the count from the group's first member and read every member's rows.
+int check_groups(const pplx_a2a_world &w) {
+  const uint32_t dp = w.dev.dp;
+  if (dp == 1) return PPLX_A2A_OK;
+  for (uint32_t g = 0; g < w.dev.G; ++g) {
+    const DispatchRank &head = w.pend_dispatch[g * dp];
+    for (uint32_t i = 1; i < dp; ++i) {
+      const DispatchRank &member = w.pend_dispatch[g * dp + i];
+      if (member.m != head.m || (member.bound_m == nullptr) != (head.bound_m == nullptr))
+        return fail(PPLX_A2A_INVALID_ARGUMENT,
+                    "ranks %u and %u share a DP group but pass %u and %u tokens (or only one of them a bound_m)",
+                    g * dp, g * dp + i, head.m, member.m);
+    }
+  }
+  return PPLX_A2A_OK;
+}
+
+// Per-rank calls of one step may arrive on different streams (the reference runs each rank's op
+// on that rank's current stream, csrc/bindings/all_to_all_ops.cpp:163,194).  The kernels go to
+// the stream of the last caller: before them it waits for what the other streams hold so far,
+// and afterwards those streams wait for the kernels, so that work enqueued on any of them after
+// the step's last call sees the outputs.
+template <typename Run>
+int run_ordered(pplx_a2a_world &w, const std::vector<void *> &streams, void *launch, Run run) {
+  bool mixed = false;
+  for (void *s : streams) mixed = mixed || s != launch;
+  if (!mixed) return run();
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  const uint32_t R = w.dev.R;
+  auto first_use = [&](uint32_t r) {
+    if (streams[r] == launch) return false;
+    for (uint32_t q = 0; q < r; ++q)
+      if (streams[q] == streams[r]) return false;
+    return true;
+  };
+  for (uint32_t r = 0; r <= R; ++r) {
+    unsigned long long session = 0;
+    int st = capture_session(r == R ? launch : streams[r], &session);
+    if (st) return st;
+    if (session != 0)
+      return fail(PPLX_A2A_INVALID_STATE, "the ranks of a captured step must call on one stream");
+  }
+  for (uint32_t r = 0; r < R; ++r) {
+    if (!first_use(r)) continue;
+    HIP_TRY(hipEventRecord(w.rank_events[r], (hipStream_t)streams[r]));
+    HIP_TRY(hipStreamWaitEvent((hipStream_t)launch, w.rank_events[r], 0));
+  }
+  int st = run();
+  if (st) return st;
+  HIP_TRY(hipEventRecord(w.done_event, (hipStream_t)launch));
+  for (uint32_t r = 0; r < R; ++r) {
+    if (first_use(r)) HIP_TRY(hipStreamWaitEvent((hipStream_t)streams[r], w.done_event, 0));
+  }
+  return PPLX_A2A_OK;
+}
+
 int run_dispatch(pplx_a2a_world &w, void *stream) {
+  int st = check_groups(w);
+  if (st) return st;
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   unsigned long long session = 0;
-  int st = capture_session(stream, &session);
+  st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
+  ProfilerRange range("dispatch");
   if (w.dev.R <= kInlineRanks) {
     LAUNCH_TRY(launch_dispatch(w.dev, w.pend_dispatch.data(), pick_vector_of(w), stream));
     return PPLX_A2A_OK;
@@ -311,6 +417,7 @@ int run_combine(pplx_a2a_world &w, void *stream) {
   int st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_combine, w.bound_combine_valid);
+  ProfilerRange range("combine");
   if (w.dev.R <= kInlineRanks) {
     LAUNCH_TRY(launch_combine(w.dev, w.pend_combine.data(), w.combine_in_dtype, w.combine_out_dtype,
                               stream));
@@ -339,74 +446,80 @@ void free_split(pplx_a2a_world &w) {
   (void)hipFree(sp.stage_y);
   sp = SplitDev{};
   w.split_ready = false;
+  w.split_y_elem_bytes = 0;
 }
 
-// Allocates the staging of split mode on first use (never inside a stream capture).
-int ensure_split(pplx_a2a_world &w, void *stream) {
-  if (w.split_ready) return PPLX_A2A_OK;
-  unsigned long long session = 0;
-  int st = capture_session(stream, &session);
-  if (st) return st;
-  if (session != 0)
-    return fail(PPLX_A2A_INVALID_STATE,
-                "the first split send/recv call allocates staging and cannot be captured; "
-                "run one eager step first");
+// Allocates (or widens) the staging of split mode.  Never part of a dispatch / combine call.
+int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
+  if (y_elem_bytes != 0 && y_elem_bytes != 2 && y_elem_bytes != 4)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "expert_y_elem_bytes must be 0, 2 or 4");
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   const WorldDev &d = w.dev;
   SplitDev &sp = w.split;
-  sp.token_stride = (uint32_t)round_up((uint64_t)d.Hb + 4ull * d.S + 4, 16);
-  const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
-  sp.tiles_per_group = (uint32_t)((d.M + tile_tokens - 1) / tile_tokens);
   const size_t pairs = (size_t)d.G * d.M * d.K;
-  struct Alloc {
-    void **ptr;
-    size_t bytes;
-  } allocs[] = {
-      {reinterpret_cast<void **>(&sp.stage_x), pairs * sp.token_stride},
-      {reinterpret_cast<void **>(&sp.gtile_cnt), sizeof(uint32_t) * (size_t)d.G * sp.tiles_per_group * d.E},
-      {reinterpret_cast<void **>(&sp.gslot), sizeof(uint32_t) * pairs},
-      {reinterpret_cast<void **>(&sp.gexp), sizeof(uint32_t) * pairs},
-      {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.G * d.E},
-      {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.G * d.E},
-      {reinterpret_cast<void **>(&sp.gbase), sizeof(uint32_t) * (size_t)d.G * d.E},
-      {reinterpret_cast<void **>(&sp.gntok), sizeof(uint32_t) * (size_t)d.G},
-  };
-  for (const Alloc &a : allocs) {
-    hipError_t err = hipMalloc(a.ptr, a.bytes);
-    if (err == hipSuccess) err = hipMemset(*a.ptr, 0, a.bytes);
-    if (err != hipSuccess) {
-      free_split(w);
-      return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of split-mode staging failed: %s", a.bytes,
-                  hipGetErrorString(err));
+  if (!w.split_ready) {
+    if (w.n_arrived_dispatch != 0 || w.n_arrived_combine != 0)
+      return fail(PPLX_A2A_INVALID_STATE, "a step is being assembled");
+    sp.token_stride = (uint32_t)round_up((uint64_t)d.Hb + 4ull * d.S + 4, 16);
+    // One group's SEND routes max_num_tokens tokens: a single tile when they fit one workgroup.
+    sp.tile_chunks = 1;
+    while (sp.tile_chunks < 16 && (uint64_t)sp.tile_chunks * kWave < d.M) sp.tile_chunks *= 2;
+    while (sp.tile_chunks > 1 && route_lds_bytes(d.E, sp.tile_chunks) > 65536u) sp.tile_chunks /= 2;
+    const uint64_t tile_tokens = (uint64_t)sp.tile_chunks * kWave;
+    sp.tiles_per_group = (uint32_t)((d.M + tile_tokens - 1) / tile_tokens);
+    struct Alloc {
+      void **ptr;
+      size_t bytes;
+    } allocs[] = {
+        {reinterpret_cast<void **>(&sp.stage_x), pairs * sp.token_stride},
+        {reinterpret_cast<void **>(&sp.gtile_cnt), sizeof(uint32_t) * (size_t)d.G * sp.tiles_per_group * d.E},
+        {reinterpret_cast<void **>(&sp.gslot), sizeof(uint32_t) * pairs},
+        {reinterpret_cast<void **>(&sp.gexp), sizeof(uint32_t) * pairs},
+        {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.G * d.E},
+        {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.G * d.E},
+        {reinterpret_cast<void **>(&sp.gbase), sizeof(uint32_t) * (size_t)d.G * d.E},
+        {reinterpret_cast<void **>(&sp.gntok), sizeof(uint32_t) * (size_t)d.G},
+    };
+    for (const Alloc &a : allocs) {
+      hipError_t err = hipMalloc(a.ptr, a.bytes);
+      if (err == hipSuccess) err = hipMemset(*a.ptr, 0, a.bytes);
+      if (err != hipSuccess) {
+        free_split(w);
+        return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of split-mode staging failed: %s", a.bytes,
+                    hipGetErrorString(err));
+      }
     }
+    w.dsend.assign(d.R, 0);
+    w.drecv.assign(d.R, 0);
+    w.csend.assign(d.R, 0);
+    w.crecv.assign(d.R, 0);
+    w.group_routed.assign(d.G, 0);
+    w.split_ready = true;
   }
-  w.dsend.assign(d.R, 0);
-  w.drecv.assign(d.R, 0);
-  w.csend.assign(d.R, 0);
-  w.crecv.assign(d.R, 0);
-  w.split_ready = true;
+  if (y_elem_bytes > w.split_y_elem_bytes) {
+    if (w.n_csend != 0 || w.n_crecv != 0)
+      return fail(PPLX_A2A_INVALID_STATE, "a split combine step is in flight");
+    // stage_y holds one expert_y row per (token, pick)
+    HIP_TRY(hipDeviceSynchronize());
+    (void)hipFree(sp.stage_y);
+    sp.stage_y = nullptr;
+    w.split_y_elem_bytes = 0;
+    const size_t bytes = pairs * (size_t)d.H * y_elem_bytes;
+    hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_y), bytes);
+    if (err != hipSuccess)
+      return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of combine staging failed: %s", bytes,
+                  hipGetErrorString(err));
+    w.split_y_elem_bytes = y_elem_bytes;
+  }
   return PPLX_A2A_OK;
 }
 
-// stage_y holds one expert_y row per (token, pick); sized for the widest dtype seen so far.
-int ensure_stage_y(pplx_a2a_world &w, int in_dtype, void *stream) {
-  const uint64_t row_bytes = (uint64_t)w.dev.H * dtype_size(in_dtype);
-  SplitDev &sp = w.split;
-  if (sp.stage_y && sp.y_row_bytes == row_bytes) return PPLX_A2A_OK;
-  unsigned long long session = 0;
-  int st = capture_session(stream, &session);
-  if (st) return st;
-  if (session != 0)
+int need_split(const pplx_a2a_world &w, uint32_t y_elem_bytes) {
+  if (!w.split_ready || w.split_y_elem_bytes < y_elem_bytes)
     return fail(PPLX_A2A_INVALID_STATE,
-                "the first split combine of a dtype allocates staging and cannot be captured");
-  HIP_TRY(hipDeviceSynchronize());
-  (void)hipFree(sp.stage_y);
-  sp.stage_y = nullptr;
-  const size_t bytes = (size_t)w.dev.G * w.dev.M * w.dev.K * row_bytes;
-  hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_y), bytes);
-  if (err != hipSuccess)
-    return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of combine staging failed: %s", bytes,
-                hipGetErrorString(err));
-  sp.y_row_bytes = row_bytes;
+                "send / recv calls need staging for %u-byte expert_y elements: call "
+                "pplx_a2a_world_reserve_split first (dispatch and combine never allocate)", y_elem_bytes);
   return PPLX_A2A_OK;
 }
 
@@ -415,14 +528,21 @@ int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, in
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   if (w.n_arrived_dispatch != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv dispatch step is still being assembled");
-  int st = ensure_split(w, stream);
+  int st = need_split(w, 0);
   if (st) return st;
   const uint32_t R = w.dev.R;
+  ProfilerRange range(mode == PPLX_A2A_SPLIT_SEND ? "dispatch send" : "dispatch recv");
   if (mode == PPLX_A2A_SPLIT_SEND) {
     if (w.n_drecv != 0)
       return fail(PPLX_A2A_INVALID_STATE,
                   "rank %u: dispatch SEND of the next step before every rank's RECV of this one", rank);
     if (w.dsend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called dispatch SEND twice", rank);
+    // The first member of a DP group to send routes the group (its members hold the same tokens).
+    const uint32_t g = rank / w.dev.dp;
+    if (!w.group_routed[g]) {
+      LAUNCH_TRY(launch_split_route(w.dev, w.split, row, rank, pick_vector_for(w.dev.K, row.indices), stream));
+      w.group_routed[g] = 1;
+    }
     LAUNCH_TRY(launch_split_dispatch_send(w.dev, w.split, row, rank, stream));
     w.dsend[rank] = 1;
     ++w.n_dsend;
@@ -438,6 +558,7 @@ int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, in
   if (++w.n_drecv == R) {
     std::fill(w.dsend.begin(), w.dsend.end(), 0);
     std::fill(w.drecv.begin(), w.drecv.end(), 0);
+    std::fill(w.group_routed.begin(), w.group_routed.end(), 0);
     w.n_dsend = w.n_drecv = 0;
   }
   return PPLX_A2A_OK;
@@ -449,9 +570,10 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   if (w.n_arrived_combine != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv combine step is still being assembled");
-  int st = ensure_split(w, stream);
+  int st = need_split(w, (uint32_t)dtype_size(in_dtype));
   if (st) return st;
   const uint32_t R = w.dev.R;
+  ProfilerRange range(mode == PPLX_A2A_SPLIT_SEND ? "combine send" : "combine recv");
   if (mode == PPLX_A2A_SPLIT_SEND) {
     if (w.n_crecv != 0)
       return fail(PPLX_A2A_INVALID_STATE,
@@ -459,9 +581,8 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
     if (w.csend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine SEND twice", rank);
     if (w.n_csend != 0 && w.split_in_dtype != in_dtype)
       return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
-    st = ensure_stage_y(w, in_dtype, stream);
-    if (st) return st;
     w.split_in_dtype = in_dtype;
+    w.split.y_row_bytes = (uint64_t)w.dev.H * dtype_size(in_dtype);
     LAUNCH_TRY(launch_split_combine_send(w.dev, w.split, row, rank, in_dtype, stream));
     w.csend[rank] = 1;
     ++w.n_csend;
@@ -501,7 +622,12 @@ extern "C" {
 
 const char *pplx_a2a_last_error(void) { return g_last_error.c_str(); }
 
-const char *pplx_a2a_version(void) { return "0.1.0"; }
+const char *pplx_a2a_version(void) { return "0.2.0"; }
+
+#ifndef PPLX_A2A_SOURCE_ID
+#define PPLX_A2A_SOURCE_ID "unknown"
+#endif
+const char *pplx_a2a_build_id(void) { return PPLX_A2A_SOURCE_ID; }
 
 int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_world_t **out) {
   if (!cfg || !out) return fail(PPLX_A2A_INVALID_ARGUMENT, "cfg / out is NULL");
@@ -530,13 +656,19 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
   d.H = (uint32_t)cfg->hidden_dim;
   d.Hb = (uint32_t)cfg->hidden_dim_bytes;
   d.S = (uint32_t)(cfg->hidden_dim_scale_bytes / 4);
-  // Largest power-of-two chunk count (<= 16) whose LDS tables fit 64 KiB.
-  d.tile_chunks = 16;
+  // Routing tiles of a whole step: small enough that a step has a few hundred of them (a tile
+  // is one workgroup, and routing is a chain of short launches that only parallelism shortens),
+  // at most 16 chunks of 64 tokens, and such that the LDS tables fit 64 KiB.
+  const uint64_t step_chunks = ((uint64_t)d.G * d.M + kWave - 1) / kWave;
+  d.tile_chunks = 1;
+  while (d.tile_chunks < 16 && step_chunks / d.tile_chunks > 256) d.tile_chunks *= 2;
   while (d.tile_chunks > 1 && route_lds_bytes(d.E, d.tile_chunks) > 65536u) d.tile_chunks /= 2;
   const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
   d.num_tiles = (uint32_t)(((uint64_t)d.G * d.M + tile_tokens - 1) / tile_tokens);
 
   auto cleanup = [&]() {
+    for (hipEvent_t ev : w->rank_events) (void)hipEventDestroy(ev);
+    if (w->done_event) (void)hipEventDestroy(w->done_event);
     (void)hipFree(d.drank);
     (void)hipFree(d.crank);
     (void)hipFree(d.tile_cnt);
@@ -563,6 +695,18 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
                   hipGetErrorString(err));
     }
   }
+  // Events that order per-rank calls made on different streams (no timing: they only fence).
+  for (uint32_t r = 0; r <= d.R; ++r) {
+    hipEvent_t ev = nullptr;
+    const hipError_t err = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+    if (err != hipSuccess) {
+      cleanup();
+      return fail(PPLX_A2A_HIP_ERROR, "hipEventCreateWithFlags failed: %s", hipGetErrorString(err));
+    }
+    if (r < d.R) w->rank_events.push_back(ev); else w->done_event = ev;
+  }
+  w->stream_dispatch.assign(d.R, nullptr);
+  w->stream_combine.assign(d.R, nullptr);
   w->pend_dispatch.assign(d.R, DispatchRank{});
   w->pend_combine.assign(d.R, CombineRank{});
   w->bound_dispatch.assign(d.R, DispatchRank{});
@@ -579,6 +723,8 @@ int pplx_a2a_world_destroy(pplx_a2a_world_t *w) {
     return fail(PPLX_A2A_INVALID_STATE, "%d rank handle(s) still attached to the world", w->attached);
   DeviceScope scope(w->device);
   (void)hipDeviceSynchronize();
+  for (hipEvent_t ev : w->rank_events) (void)hipEventDestroy(ev);
+  if (w->done_event) (void)hipEventDestroy(w->done_event);
   (void)hipFree(w->dev.drank);
   (void)hipFree(w->dev.crank);
   (void)hipFree(w->dev.tile_cnt);
@@ -645,10 +791,11 @@ int pplx_a2a_dispatch(pplx_a2a_t *h, const pplx_a2a_dispatch_args_t *args, int s
     return fail(PPLX_A2A_INVALID_STATE,
                 "rank %u called dispatch twice before the other ranks of the step", h->rank);
   w.pend_dispatch[h->rank] = row;
+  w.stream_dispatch[h->rank] = stream;
   w.arrived_dispatch[h->rank] = 1;
   if (++w.n_arrived_dispatch < w.dev.R) return PPLX_A2A_OK;
   reset_dispatch_arrivals(w);
-  return run_dispatch(w, stream);
+  return run_ordered(w, w.stream_dispatch, stream, [&] { return run_dispatch(w, stream); });
 }
 
 int pplx_a2a_combine(pplx_a2a_t *h, const pplx_a2a_combine_args_t *args, int split_mode,
@@ -675,13 +822,14 @@ int pplx_a2a_combine(pplx_a2a_t *h, const pplx_a2a_combine_args_t *args, int spl
   w.combine_in_dtype = args->in_dtype;
   w.combine_out_dtype = args->out_dtype;
   w.pend_combine[h->rank] = row;
+  w.stream_combine[h->rank] = stream;
   w.arrived_combine[h->rank] = 1;
   if (++w.n_arrived_combine < w.dev.R) return PPLX_A2A_OK;
   const int in_dt = w.combine_in_dtype, out_dt = w.combine_out_dtype;
   reset_combine_arrivals(w);
   w.combine_in_dtype = in_dt;
   w.combine_out_dtype = out_dt;
-  return run_combine(w, stream);
+  return run_ordered(w, w.stream_combine, stream, [&] { return run_combine(w, stream); });
 }
 
 int pplx_a2a_world_dispatch(pplx_a2a_world_t *w, const pplx_a2a_dispatch_args_t *per_rank,
@@ -712,6 +860,12 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *w, const pplx_a2a_combine_args_t *p
   w->combine_in_dtype = per_rank[0].in_dtype;
   w->combine_out_dtype = per_rank[0].out_dtype;
   return run_combine(*w, stream);
+}
+
+int pplx_a2a_world_reserve_split(pplx_a2a_world_t *w, uint32_t expert_y_elem_bytes) {
+  if (!w) return fail(PPLX_A2A_INVALID_ARGUMENT, "world is NULL");
+  std::lock_guard<std::mutex> lock(w->mu);
+  return reserve_split(*w, expert_y_elem_bytes);
 }
 
 int pplx_a2a_world_faults(pplx_a2a_world_t *w, void *stream, uint32_t *out_bits) {

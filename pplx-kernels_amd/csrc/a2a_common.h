@@ -166,6 +166,74 @@ __device__ __forceinline__ uint32_t dispatch_group_tokens(const WorldDev &w, con
   return n < w.M ? n : w.M;
 }
 
+// True when the group's bound_m asks for more tokens than dispatch_group_tokens() lets through
+// (the reference asserts numSendTokens <= maxNumTokens, csrc/all_to_all/intranode_dispatch.cu:65).
+template <class DT>
+__device__ __forceinline__ bool dispatch_group_overflows(const WorldDev &w, const DT &tab, uint32_t g) {
+  const DispatchRank &r = tab.at(g * w.dp);
+  if (!r.bound_m) return r.m > w.M;
+  const uint32_t n = *as_global(r.bound_m);
+  return n > r.m || n > w.M;
+}
+
+// PV consecutive expert ids as one register value (PV = 1, 2 or 4).
+template <int PV> struct PickVector;
+template <> struct PickVector<1> {
+  typedef uint32_t type;
+  static __device__ __forceinline__ uint32_t at(type x, int) { return x; }
+};
+template <> struct PickVector<2> {
+  typedef uint32_t type __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
+};
+template <> struct PickVector<4> {
+  typedef u32x4 type;
+  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
+};
+
+// What a pass over the picks of one token found: bit k of `marked` is set when fn returned a
+// non-zero code for pick k, `codes` is the OR of all codes.
+struct PickMarks {
+  unsigned long long marked;
+  uint32_t codes;
+};
+
+// Calls fn(k, expert) for the K picks at `idx` in order and collects the codes it returns.  The
+// picks are fetched PV at a time (K % PV == 0, idx aligned to the vector) and up to four vectors
+// are in flight at once, so a top-8 row of picks costs one trip to memory instead of eight.
+template <int PV, class Fn>
+__device__ __forceinline__ PickMarks for_each_pick(const PPLX_GLOBAL uint32_t *idx, uint32_t K, Fn &&fn) {
+  typedef PickVector<PV> Vec;
+  typedef typename Vec::type vec_t;
+  const PPLX_GLOBAL vec_t *p = reinterpret_cast<const PPLX_GLOBAL vec_t *>(idx);
+  const uint32_t vectors = K / PV;
+  PickMarks marks{0ull, 0u};
+  auto visit = [&](uint32_t j, vec_t x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < PV; ++u) {
+      const uint32_t code = fn(j * PV + u, Vec::at(x, u));
+      marks.codes |= code;
+      marks.marked |= (unsigned long long)(code != 0) << (j * PV + u);
+    }
+  };
+  uint32_t j = 0;
+  for (; j + 4 <= vectors; j += 4) {
+    const vec_t a = p[j], b = p[j + 1], c = p[j + 2], d = p[j + 3];
+    visit(j, a);
+    visit(j + 1, b);
+    visit(j + 2, c);
+    visit(j + 3, d);
+  }
+  if (vectors - j >= 2) {
+    const vec_t a = p[j], b = p[j + 1];
+    visit(j, a);
+    visit(j + 1, b);
+    j += 2;
+  }
+  if (j < vectors) visit(j, p[j]);
+  return marks;
+}
+
 __device__ __forceinline__ uint32_t combine_rank_tokens(const WorldDev &w, const CombineRank &c) {
   uint32_t n = c.bound_m ? *as_global(c.bound_m) : c.m;
   n = n < c.m ? n : c.m;

@@ -17,6 +17,8 @@ constexpr uint32_t kInvalidSlot = 0xffffffffu;
 constexpr uint32_t kFaultRowDropped = 1u;   // slot >= out_expert_x rows
 constexpr uint32_t kFaultBadExpert = 2u;    // index >= num_experts
 constexpr uint32_t kFaultBadSlot = 4u;      // combine slot >= expert_y rows
+constexpr uint32_t kFaultDuplicateExpert = 8u;   // an expert id repeated inside one token was dropped
+constexpr uint32_t kFaultTooManyTokens = 16u;    // bound_m > max_num_tokens (or > rows) was clamped
 
 struct alignas(16) DispatchRank {
   int32_t *out_num_tokens;
@@ -68,11 +70,12 @@ struct WorldDev {
   uint32_t H;        // elements per row
   uint32_t Hb;       // bytes per dispatched row
   uint32_t S;        // fp32 scales per row
-  uint32_t tile_chunks;  // 64-token chunks per routing tile
+  uint32_t tile_chunks;  // 64-token chunks per routing tile of a whole-step dispatch
   uint32_t num_tiles;    // ceil(G * M / (64 * tile_chunks))
   DispatchRank *drank;   // [R]
   CombineRank *crank;    // [R]
-  uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile
+  uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile; after route_scan the
+                         // tokens routed to e in all earlier tiles
   uint32_t *slot_map;    // [G * M][K] row of (token, pick) inside its expert
   uint32_t *faults;      // [1] sticky fault bits
 };
@@ -81,6 +84,8 @@ struct WorldDev {
 struct RouteSpan {
   uint32_t v_begin;       // first virtual token (tiles are counted from here)
   uint32_t v_count;       // virtual tokens covered
+  uint32_t tile_chunks;   // 64-token chunks per tile (one workgroup)
+  uint32_t pick_vector;   // expert ids one load may fetch (4, 2 or 1)
   uint32_t *tile_cnt;     // [tiles][E]
   uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
   // split mode only (one DP group per launch):
@@ -99,6 +104,7 @@ struct RouteSpan {
 struct SplitDev {
   uint8_t *stage_x;        // [G][M * K rows][token_stride]
   uint32_t token_stride;   // round_up(Hb + 4 S + 4, 16)
+  uint32_t tile_chunks;    // 64-token chunks per routing tile of one group's SEND
   uint32_t tiles_per_group;
   uint32_t *gtile_cnt;     // [G][tiles_per_group][E]
   uint32_t *gslot;         // [G * M][K] row of a pair inside its (group, expert) run
@@ -149,6 +155,10 @@ int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
 // Split mode phases of one rank (`row` holds that rank's arguments of the call).
+// Routes the DP group of `rank` from that rank's indices (the members of a group hold the same
+// tokens, so the first member to send does it for the group); then every member packs its share.
+int launch_split_route(const WorldDev &w, const SplitDev &sp, const DispatchRank &row, uint32_t rank,
+                       uint32_t pick_vector, void *stream);
 int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
                                uint32_t rank, void *stream);
 int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,

@@ -82,21 +82,6 @@ struct LdsDispatch {
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
 
-// PV consecutive expert ids as one register value (PV = 1, 2 or 4).
-template <int PV> struct PickVector;
-template <> struct PickVector<1> {
-  typedef uint32_t type;
-  static __device__ __forceinline__ uint32_t at(type x, int) { return x; }
-};
-template <> struct PickVector<2> {
-  typedef uint32_t type __attribute__((ext_vector_type(2)));
-  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
-};
-template <> struct PickVector<4> {
-  typedef u32x4 type;
-  static __device__ __forceinline__ uint32_t at(type x, int u) { return x[u]; }
-};
-
 // Reads the picks of virtual tokens [0, v_own_end), one thread per token and PV picks per load
 // (K % PV == 0 and every indices pointer aligned to the vector: the host checks both): those
 // of tokens before v_own go into the LDS histogram, those of the workgroup's own tokens
@@ -150,15 +135,25 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
         if (second) keep[PV + u] = Vec::at(b, u);
       }
     } else if (f.t < f.n) {
+      // An earlier token: every expert it names counts once (a repeat takes no row).  The
+      // picks of this call are compared in registers; those of earlier calls for the same
+      // token (top-k beyond two vectors) are read again.
+      uint32_t e[2 * PV];
 #pragma unroll
       for (int u = 0; u < PV; ++u) {
-        const uint32_t e = Vec::at(a, u);
-        if (e < w.E) atomicAdd(&hist[e], 1u);
+        e[u] = Vec::at(a, u);
+        e[PV + u] = second ? Vec::at(b, u) : w.E;
       }
 #pragma unroll
-      for (int u = 0; u < PV; ++u) {
-        const uint32_t e = Vec::at(b, u);
-        if (second && e < w.E) atomicAdd(&hist[e], 1u);
+      for (int u = 0; u < 2 * PV; ++u) {
+        bool counts = e[u] < w.E;
+#pragma unroll
+        for (int p = 0; p < u; ++p) counts = counts && e[p] != e[u];
+        if (counts && j != 0) {
+          const PPLX_GLOBAL uint32_t *before = reinterpret_cast<const PPLX_GLOBAL uint32_t *>(f.idx);
+          for (uint32_t p = 0; p < j * PV; ++p) counts = counts && before[p] != e[u];
+        }
+        if (counts) atomicAdd(&hist[e[u]], 1u);
       }
     }
   };
@@ -210,7 +205,8 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   uint32_t *ntok = hist + w.E;                                                 // [G]
   uint32_t *own_e = ntok + w.G;                                                // [own_pairs]
   for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) hist[e] = 0;
-  if constexpr (kStaged) __syncthreads();
+  // Orders the zeroing (and the staged table) before the first counter update of any wave.
+  __syncthreads();
   const LdsDispatch staged{reinterpret_cast<const DispatchRank *>(lds_u64)};
   auto rows = [&]() -> decltype(auto) {
     if constexpr (kStaged) return (staged); else return (tab);
@@ -262,25 +258,32 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
     read_picks<1, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
   }
   if (counts_group) {
-    uint32_t n = counted_bound ? counted_loaded : counted.m;
-    n = n < counted.m ? n : counted.m;
-    ntok[threadIdx.x] = n < w.M ? n : w.M;
+    const uint32_t asked = counted_bound ? counted_loaded : counted.m;
+    uint32_t n = asked < counted.m ? asked : counted.m;
+    n = n < w.M ? n : w.M;
+    ntok[threadIdx.x] = n;
+    if (n != asked && blockIdx.x == 0) atomicOr(w.faults, kFaultTooManyTokens);
   }
   for (uint32_t g = threadIdx.x + kFusedThreads; g < w.G; g += kFusedThreads) {
     ntok[g] = dispatch_group_tokens(w, rows(), g);
+    if (blockIdx.x == 0 && dispatch_group_overflows(w, rows(), g)) atomicOr(w.faults, kFaultTooManyTokens);
   }
   __syncthreads();
 
-  // 3. own slots, token by token (the experts of one token are distinct: no two threads of a
-  // round share a counter), then the destinations
+  // 3. own slots, token by token (a pick that repeats an earlier expert of its token takes no
+  // row, so no two threads of a round share a counter), then the destinations
   const bool pick_live = pick_exists && pick_t < ntok[pick_g];
   const uint32_t pick_e = pick_exists ? own_e[threadIdx.x] : w.E;
+  bool pick_repeats = false;
+  if (pick_live) {
+    for (uint32_t k = 0; k < pick_k; ++k) pick_repeats = pick_repeats || own_e[threadIdx.x - pick_k + k] == pick_e;
+  }
   uint32_t pick_slot = kInvalidSlot;
   // (when all pick threads sit in one wave the hardware keeps its LDS accesses in order by
   // itself; the fence keeps the compiler from moving them across the rounds)
   const bool one_wave = own_pairs <= kWave;
   for (uint32_t j = 0; j < tokens_per_block; ++j) {
-    if (pick_live && pick_j == j && pick_e < w.E) {
+    if (pick_live && pick_j == j && pick_e < w.E && !pick_repeats) {
       pick_slot = hist[pick_e];
       hist[pick_e] = pick_slot + 1;
     }
@@ -295,7 +298,11 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
     if (pick_live) {
       d = resolve_destination(w, rows(), pick_e, pick_slot, true);
       as_global(w.slot_map)[(size_t)pick_v * w.K + pick_k] = pick_slot;
-      if (pick_e >= w.E) atomicOr(w.faults, kFaultBadExpert);
+      if (pick_e >= w.E) {
+        atomicOr(w.faults, kFaultBadExpert);
+      } else if (pick_repeats) {
+        atomicOr(w.faults, kFaultDuplicateExpert);
+      }
     }
     dst_row[threadIdx.x] = d.row;
     dst_scale[threadIdx.x] = d.scale;
@@ -447,6 +454,8 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hi
   RouteSpan span{};
   span.v_begin = 0;
   span.v_count = w.G * w.M;
+  span.tile_chunks = w.tile_chunks;
+  span.pick_vector = pick_vector;
   span.tile_cnt = w.tile_cnt;
   span.slot_out = w.slot_map;
   int err = launch_route_t<DT, false>(w, tab, span, s);

@@ -7,106 +7,163 @@ namespace {
 
 // ---------------------------------------------------------------------------
 // Routing.  Virtual token v = g * M + t enumerates (DP group asc, token asc),
-// the order in which the reference test appends to expert_token_from.  A tile
-// is tile_chunks consecutive chunks of 64 virtual tokens.
-// ---------------------------------------------------------------------------
+// the order in which the reference test appends to expert_token_from
+// (tests/test_all_to_all.py:113-120).  A chunk is 64 consecutive virtual tokens
+// (one wavefront, one token per lane), a tile is span.tile_chunks chunks (one
+// workgroup).  Per chunk and expert a 64-bit mask in LDS holds one bit per token
+// routed to the expert (ds_or_b64); a token's row inside the expert is
+//     rows of earlier tiles + rows of earlier chunks of the tile + popc(mask & lanes below).
+// Three launches when a span has more than one tile, one otherwise:
+//   route_count   per tile: rows per expert                      -> tile_cnt[tile][e]
+//   route_scan    per expert: exclusive prefix over the tiles    -> tile_cnt[tile][e], totals
+//   route_slots   per tile: the masks again, slots               -> slot map
+// An expert id repeated inside one token sets its bit once: the repeat takes no row, is not
+// counted, and is reported (kFaultDuplicateExpert).
+//
 // SPLIT = false: one launch routes every DP group and writes out_expert_num_tokens of the
 // owning ranks.  SPLIT = true: the launch routes the span of one DP group from the calling
 // rank's indices alone and leaves group-local results (slot inside (group, expert), expert of
 // each pair, rows per expert and their exclusive prefix over experts) for the later phases.
-template <class DT>
-__global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpan span) {
-  extern __shared__ uint32_t lds_hist[];
-  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_hist[e] = 0;
-  __syncthreads();
+// ---------------------------------------------------------------------------
 
+// The token of this thread: which group and sender, whether its row of picks exists, and the
+// loads that decide whether it is live (issued together with the picks by the callers).
+struct RouteToken {
+  uint32_t v, g, t;
+  bool in_span;
+  bool row_exists;                 // t < m of the sender: its picks may be read
+  uint32_t n_group;                // tokens present in the group
+  const PPLX_GLOBAL uint32_t *idx; // its K picks
+};
+
+template <class DT>
+__device__ __forceinline__ RouteToken route_token(const WorldDev &w, const DT &tab, const RouteSpan &span) {
+  RouteToken r;
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  const uint32_t v = span.v_begin + i;
-  const uint32_t g = v / w.M;
-  const uint32_t t = v - g * w.M;
-  if (i < span.v_count && g < w.G && t < dispatch_group_tokens(w, tab, g)) {
-    const PPLX_GLOBAL uint32_t *idx = as_global(tab.at(g * w.dp + t % w.dp).indices) + (size_t)t * w.K;
-    for (uint32_t k = 0; k < w.K; ++k) {
-      const uint32_t e = idx[k];
-      if (e < w.E) atomicAdd(&lds_hist[e], 1u);
-    }
-  }
-  __syncthreads();
-  uint32_t *out = span.tile_cnt + (size_t)blockIdx.x * w.E;
-  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) out[e] = lds_hist[e];
+  r.v = span.v_begin + i;
+  r.g = r.v / w.M;
+  r.t = r.v - r.g * w.M;
+  r.in_span = i < span.v_count && r.g < w.G;
+  const DispatchRank &src = tab.at(r.in_span ? r.g * w.dp + r.t % w.dp : 0);
+  r.row_exists = r.in_span && r.t < src.m;
+  r.n_group = r.in_span ? dispatch_group_tokens(w, tab, r.g) : 0;
+  r.idx = as_global(src.indices) + (size_t)r.t * w.K;
+  return r;
 }
 
-template <class DT, bool SPLIT>
-__global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpan span) {
-  // LDS: mask[chunks][E] (one bit per token of the chunk routed to e),
-  //      then base[chunks][E] (rows of e taken before the chunk starts).
+template <class DT, int PV>
+__global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpan span) {
   extern __shared__ unsigned long long lds_mask[];
-  const uint32_t chunks = w.tile_chunks;
-  uint32_t *lds_base = reinterpret_cast<uint32_t *>(lds_mask + (size_t)chunks * w.E);
-
+  const uint32_t chunks = span.tile_chunks;
   for (uint32_t i = threadIdx.x; i < chunks * w.E; i += blockDim.x) lds_mask[i] = 0ull;
-  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_base[e] = 0;
   __syncthreads();
-
-  // Rows taken by earlier tiles, summed per expert into lds_base[0][e] by the whole workgroup:
-  // the counts are fetched kTileLoads at a time so that their latencies overlap each other and
-  // the index loads below (one thread per expert walking the tiles would pay one L2 round trip
-  // per tile).
-  {
-    constexpr uint32_t kTileLoads = 8;
-    const uint32_t total = blockIdx.x * w.E;
-    for (uint32_t first = threadIdx.x; first < total; first += blockDim.x * kTileLoads) {
-      uint32_t rows[kTileLoads];
-#pragma unroll
-      for (uint32_t u = 0; u < kTileLoads; ++u) {
-        const uint32_t j = first + u * blockDim.x;
-        rows[u] = j < total ? span.tile_cnt[j] : 0u;
-      }
-#pragma unroll
-      for (uint32_t u = 0; u < kTileLoads; ++u) {
-        if (rows[u]) atomicAdd(&lds_base[(first + u * blockDim.x) % w.E], rows[u]);
-      }
-    }
-  }
 
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t chunk = threadIdx.x / kWave;
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  const uint32_t v = span.v_begin + i;
-  const uint32_t g = v / w.M;
-  const uint32_t t = v - g * w.M;
-  const bool in_span = i < span.v_count && g < w.G;
-  const uint32_t n_group = in_span ? dispatch_group_tokens(w, tab, g) : 0;
-  const bool live = in_span && t < n_group;
-  const PPLX_GLOBAL uint32_t *idx = nullptr;
-  bool bad_expert = false;
-  if (live) {
-    idx = as_global(tab.at(g * w.dp + t % w.dp).indices) + (size_t)t * w.K;
-    for (uint32_t k = 0; k < w.K; ++k) {
-      const uint32_t e = idx[k];
-      if (e < w.E) {
-        atomicOr(&lds_mask[(size_t)chunk * w.E + e], 1ull << lane);
-      } else {
-        bad_expert = true;
-      }
+  const RouteToken tok = route_token(w, tab, span);
+  // (the picks are fetched whenever their row exists, behind the group's token count and not
+  // after it: one trip to memory instead of two)
+  if (tok.row_exists) {
+    const bool live = tok.t < tok.n_group;
+    for_each_pick<PV>(tok.idx, w.K, [&](uint32_t, uint32_t e) __attribute__((always_inline)) {
+      if (live && e < w.E) atomicOr(&lds_mask[(size_t)chunk * w.E + e], 1ull << lane);
+      return 0u;
+    });
+  }
+  __syncthreads();
+  uint32_t *out = span.tile_cnt + (size_t)blockIdx.x * w.E;
+  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
+    uint32_t rows = 0;
+    for (uint32_t c = 0; c < chunks; ++c) rows += __popcll(lds_mask[(size_t)c * w.E + e]);
+    out[e] = rows;
+  }
+}
+
+// One wavefront per expert: tile_cnt[.][e] becomes its own exclusive prefix over the tiles, and
+// the total goes to out_expert_num_tokens of the owning rank
+// (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total) or, in split mode, to
+// counts_out.  Up to 256 tiles are fetched per trip to memory.
+template <class DT, bool SPLIT>
+__global__ __launch_bounds__(256) void route_scan(WorldDev w, DT tab, RouteSpan span, uint32_t tiles) {
+  const uint32_t lane = lane_id();
+  const uint32_t e = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
+  if (e >= w.E) return;
+  constexpr uint32_t kBatch = 4;
+  uint32_t carry = 0;
+  for (uint32_t t0 = 0; t0 < tiles; t0 += kBatch * kWave) {
+    uint32_t rows[kBatch];
+#pragma unroll
+    for (uint32_t b = 0; b < kBatch; ++b) {
+      const uint32_t t = t0 + b * kWave + lane;
+      rows[b] = t < tiles ? span.tile_cnt[(size_t)t * w.E + e] : 0u;
     }
+#pragma unroll
+    for (uint32_t b = 0; b < kBatch; ++b) {
+      const uint32_t t = t0 + b * kWave + lane;
+      uint32_t incl = rows[b];
+#pragma unroll
+      for (uint32_t d = 1; d < kWave; d *= 2) {
+        const uint32_t up = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += up;
+      }
+      if (t < tiles) span.tile_cnt[(size_t)t * w.E + e] = carry + incl - rows[b];
+      carry += __shfl(incl, kWave - 1, kWave);
+    }
+  }
+  if (lane == 0) {
+    if (SPLIT) {
+      span.counts_out[e] = carry;
+    } else {
+      const DispatchRank &owner = tab.at(e / w.L);
+      as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)carry;
+    }
+  }
+}
+
+// `scanned`: tile_cnt holds the rows of earlier tiles (route_scan has run); otherwise the span
+// is a single tile and this launch also writes the totals.
+template <class DT, bool SPLIT, int PV>
+__global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpan span, uint32_t scanned) {
+  // LDS: mask[chunks][E] (one bit per token of the chunk routed to e),
+  //      then base[chunks][E] (rows of e taken before the chunk starts).
+  extern __shared__ unsigned long long lds_mask[];
+  const uint32_t chunks = span.tile_chunks;
+  uint32_t *lds_base = reinterpret_cast<uint32_t *>(lds_mask + (size_t)chunks * w.E);
+
+  for (uint32_t i = threadIdx.x; i < chunks * w.E; i += blockDim.x) lds_mask[i] = 0ull;
+  {
+    const uint32_t *earlier = span.tile_cnt + (size_t)blockIdx.x * w.E;
+    for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) lds_base[e] = scanned ? earlier[e] : 0u;
+  }
+  __syncthreads();
+
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t chunk = threadIdx.x / kWave;
+  const RouteToken tok = route_token(w, tab, span);
+  const bool live = tok.row_exists && tok.t < tok.n_group;
+  // Marked picks have no row: an expert id out of range, or a repeat of an earlier pick.
+  PickMarks no_row{0ull, 0u};
+  if (tok.row_exists) {
+    no_row = for_each_pick<PV>(tok.idx, w.K, [&](uint32_t, uint32_t e) __attribute__((always_inline)) {
+      if (!live) return 0u;
+      if (e >= w.E) return kFaultBadExpert;
+      const unsigned long long bit = 1ull << lane;
+      return (atomicOr(&lds_mask[(size_t)chunk * w.E + e], bit) & bit) ? kFaultDuplicateExpert : 0u;
+    });
   }
   __syncthreads();
 
   // Per expert: running prefix over chunks, starting from the rows of earlier tiles.
-  const bool last_tile = blockIdx.x == gridDim.x - 1;
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
     uint32_t running = lds_base[e];
     for (uint32_t c = 0; c < chunks; ++c) {
       lds_base[c * w.E + e] = running;
       running += __popcll(lds_mask[(size_t)c * w.E + e]);
     }
-    if (last_tile) {
+    if (!scanned) {
       if (SPLIT) {
         span.counts_out[e] = running;
       } else {
-        // out_expert_num_tokens of the owning rank
-        // (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).
         const DispatchRank &owner = tab.at(e / w.L);
         as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
       }
@@ -116,22 +173,26 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
 
   if (live) {
     const unsigned long long below = (1ull << lane) - 1ull;
-    uint32_t *out = span.slot_out + (size_t)v * w.K;
-    for (uint32_t k = 0; k < w.K; ++k) {
-      const uint32_t e = idx[k];
+    uint32_t *out = span.slot_out + (size_t)tok.v * w.K;
+    for_each_pick<PV>(tok.idx, w.K, [&](uint32_t k, uint32_t e) __attribute__((always_inline)) {
       uint32_t slot = kInvalidSlot;
-      if (e < w.E) {
+      if (!((no_row.marked >> k) & 1ull)) {
         slot = lds_base[chunk * w.E + e] + __popcll(lds_mask[(size_t)chunk * w.E + e] & below);
       }
       out[k] = slot;
-      if (SPLIT) span.expert_out[(size_t)v * w.K + k] = e;
-    }
-    if (bad_expert) atomicOr(w.faults, kFaultBadExpert);
+      // later phases of split mode treat an id >= E as "no row"
+      if (SPLIT) span.expert_out[(size_t)tok.v * w.K + k] = slot == kInvalidSlot ? w.E : e;
+      return 0u;
+    });
+    if (no_row.codes) atomicOr(w.faults, no_row.codes);
+  }
+  if (tok.in_span && tok.t == 0 && dispatch_group_overflows(w, tab, tok.g)) {
+    atomicOr(w.faults, kFaultTooManyTokens);
   }
 
-  if (SPLIT && last_tile) {
+  if (SPLIT && blockIdx.x == gridDim.x - 1) {
     // Exclusive prefix of counts_out over experts: where each expert's rows start in the
-    // group's compact staging area.  counts_out was written by this workgroup above.
+    // group's compact staging area.  counts_out was written above or by route_scan.
     __syncthreads();
     uint32_t *scan = reinterpret_cast<uint32_t *>(lds_mask);  // blockDim entries, LDS is free now
     const uint32_t per_thread = (w.E + blockDim.x - 1) / blockDim.x;
@@ -155,18 +216,28 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
   }
 }
 
-template <class DT, bool SPLIT>
-int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
-  const uint32_t block = w.tile_chunks * kWave;
+template <class DT, bool SPLIT, int PV>
+int launch_route_pv(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
+  const uint32_t block = span.tile_chunks * kWave;
   const uint32_t tiles = (span.v_count + block - 1) / block;
+  const uint32_t lds = route_lds_bytes(w.E, span.tile_chunks);
   if (tiles > 1) {
-    hipLaunchKernelGGL(route_count<DT>, dim3(tiles), dim3(block), w.E * sizeof(uint32_t), s, w, tab, span);
+    hipLaunchKernelGGL((route_count<DT, PV>), dim3(tiles), dim3(block),
+                       span.tile_chunks * w.E * sizeof(unsigned long long), s, w, tab, span);
+    hipLaunchKernelGGL((route_scan<DT, SPLIT>), dim3((w.E + 3) / 4), dim3(256), 0, s, w, tab, span, tiles);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return (int)err;
   }
-  hipLaunchKernelGGL((route_slots<DT, SPLIT>), dim3(tiles), dim3(block),
-                     route_lds_bytes(w.E, w.tile_chunks), s, w, tab, span);
+  hipLaunchKernelGGL((route_slots<DT, SPLIT, PV>), dim3(tiles), dim3(block), lds, s, w, tab, span,
+                     tiles > 1 ? 1u : 0u);
   return (int)hipGetLastError();
+}
+
+template <class DT, bool SPLIT>
+int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
+  if (span.pick_vector == 4) return launch_route_pv<DT, SPLIT, 4>(w, tab, span, s);
+  if (span.pick_vector == 2) return launch_route_pv<DT, SPLIT, 2>(w, tab, span, s);
+  return launch_route_pv<DT, SPLIT, 1>(w, tab, span, s);
 }
 
 }  // namespace

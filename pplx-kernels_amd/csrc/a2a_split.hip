@@ -24,7 +24,8 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g
   if (t >= w.M || t % w.dp != member || t >= sp.gntok[g]) return;
   const DispatchRank &src = tab.at(0);
   const uint32_t nvec = w.Hb / 16;
-  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
+  const PPLX_GLOBAL u32x4 *row =
+      as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
   u32x4 x[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -33,16 +34,25 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g
     x[i] = row[j];
   }
   const uint32_t S = w.S;
-  const float *srow = S ? src.dp_xs + (int64_t)t * src.dp_xs_stride_row : nullptr;
+  // scale `lane` of the row; rows of more than 64 scales take the loop below
+  float sc = 0.f;
+  const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
+  if (S) sc = srow[(int64_t)(lane < S ? lane : S - 1) * src.dp_xs_stride_elem];
   uint64_t dst = 0;
   if (lane < w.K) {
     const size_t pair = ((size_t)g * w.M + t) * w.K + lane;
-    const uint32_t e = sp.gexp[pair];
-    if (e < w.E) dst = reinterpret_cast<uint64_t>(stage_row(w, sp, g, sp.goff[(size_t)g * w.E + e] + sp.gslot[pair]));
+    const uint32_t e = as_global(sp.gexp)[pair];
+    if (e < w.E) {
+      dst = reinterpret_cast<uint64_t>(
+          stage_row(w, sp, g, as_global(sp.goff)[(size_t)g * w.E + e] + as_global(sp.gslot)[pair]));
+    }
   }
 #pragma unroll
   for (int i = 0; i < NV; ++i) settle(x[i]);
+  settle(sc);
   settle(dst);
+  // The staged rows are read back by the RECV phase next: they are stored write-through so
+  // that they stay in the last-level cache when they fit there.
   for (uint32_t k = 0; k < w.K; ++k) {
     const uint64_t p = read_lane64(dst, k);
     if (p == 0) continue;
@@ -50,10 +60,11 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const uint32_t j = lane + i * kWave;
-      if (EXACT || j < nvec) out[j] = x[i];
+      if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[i], out + j);
     }
     PPLX_GLOBAL float *sout = global_ptr<float>(p + w.Hb);
-    for (uint32_t j = lane; j < S; j += kWave) sout[j] = srow[(int64_t)j * src.dp_xs_stride_elem];
+    if (lane < S) row_store<RowStore::kKeep>(sc, sout + lane);
+    for (uint32_t j = lane + kWave; j < S; j += kWave) sout[j] = srow[(int64_t)j * src.dp_xs_stride_elem];
     if (lane == 0) *global_ptr<uint32_t>(p + w.Hb + 4ull * S) = t;
   }
 }
@@ -84,7 +95,8 @@ __global__ __launch_bounds__(256) void split_finalize(WorldDev w, SplitDev sp) {
 // dispatch RECV of rank d: workgroup (local expert, group) copies that run of staged rows
 // into out_expert_x / out_expert_x_scale; blockIdx.y spreads long runs.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t d, SplitDev sp) {
+__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t d, SplitDev sp,
+                                                    uint32_t write_through) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const uint32_t el = blockIdx.x / w.G;
@@ -92,10 +104,11 @@ __global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t
   const uint32_t e = d * w.L + el;
   const DispatchRank &dst = tab.at(0);
   const size_t ge = (size_t)g * w.E + e;
-  const uint32_t count = sp.gcnt[ge], offset = sp.goff[ge], base = sp.gbase[ge];
+  const uint32_t count = as_global(sp.gcnt)[ge], offset = as_global(sp.goff)[ge], base = as_global(sp.gbase)[ge];
   if (g == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
     const size_t last = (size_t)(w.G - 1) * w.E + e;
-    dst.out_num_tokens[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)(sp.gbase[last] + sp.gcnt[last]);
+    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] =
+        (int32_t)(as_global(sp.gbase)[last] + as_global(sp.gcnt)[last]);
   }
   const uint32_t nvec = w.Hb / 16;
   const uint32_t S = w.S;
@@ -106,9 +119,9 @@ __global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t
       continue;
     }
     const uint8_t *src = stage_row(w, sp, g, offset + i);
-    const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
-    u32x4 *out = reinterpret_cast<u32x4 *>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
-                                           (int64_t)slot * dst.x_stride_row);
+    const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
+    PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
+        dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
     u32x4 x[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -116,16 +129,31 @@ __global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t
       if (!EXACT) j = j < nvec ? j : nvec - 1;
       x[v] = row[j];
     }
+    float sc = 0.f;
+    const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
+    if (S) sc = sin[lane < S ? lane : S - 1];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      const uint32_t j = lane + v * kWave;
-      if (EXACT || j < nvec) __builtin_nontemporal_store(x[v], out + j);
+    for (int v = 0; v < NV; ++v) settle(x[v]);
+    settle(sc);
+    PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
+                              (int64_t)slot * dst.xs_stride_row;
+    // same policy as the one-call dispatch: rows that fit the last-level cache stay there
+    if (write_through) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const uint32_t j = lane + v * kWave;
+        if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[v], out + j);
+      }
+      if (lane < S) row_store<RowStore::kKeep>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
+    } else {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const uint32_t j = lane + v * kWave;
+        if (EXACT || j < nvec) row_store<RowStore::kStream>(x[v], out + j);
+      }
+      if (lane < S) row_store<RowStore::kStream>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
     }
-    if (S) {
-      const float *sin = reinterpret_cast<const float *>(src + w.Hb);
-      float *sout = dst.expert_xs + (int64_t)el * dst.xs_stride_expert + (int64_t)slot * dst.xs_stride_row;
-      for (uint32_t j = lane; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
-    }
+    for (uint32_t j = lane + kWave; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
   }
 }
 
@@ -214,23 +242,31 @@ __global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, ui
 
 }  // namespace
 
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
-                               uint32_t rank, void *stream) {
+int launch_split_route(const WorldDev &w, const SplitDev &sp, const DispatchRank &row, uint32_t rank,
+                       uint32_t pick_vector, void *stream) {
   typedef SingleDispatch DT;
-  hipStream_t s = (hipStream_t)stream;
   const DT tab{row};
-  const uint32_t g = rank / w.dp, member = rank % w.dp;
+  const uint32_t g = rank / w.dp;
   RouteSpan span{};
   span.v_begin = g * w.M;
   span.v_count = w.M;
+  span.tile_chunks = sp.tile_chunks;
+  span.pick_vector = pick_vector;
   span.tile_cnt = sp.gtile_cnt + (size_t)g * sp.tiles_per_group * w.E;
   span.slot_out = sp.gslot;
   span.expert_out = sp.gexp;
   span.counts_out = sp.gcnt + (size_t)g * w.E;
   span.offsets_out = sp.goff + (size_t)g * w.E;
   span.ntok_out = sp.gntok + g;
-  int err = launch_route_t<DT, true>(w, tab, span, s);
-  if (err) return err;
+  return launch_route_t<DT, true>(w, tab, span, (hipStream_t)stream);
+}
+
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
+                               uint32_t rank, void *stream) {
+  typedef SingleDispatch DT;
+  hipStream_t s = (hipStream_t)stream;
+  const DT tab{row};
+  const uint32_t g = rank / w.dp, member = rank % w.dp;
   const uint32_t lds = 0;
   if (!row_has_register_variant(w)) {
     hipLaunchKernelGGL(split_pack_long<DT>, dim3(w.M), dim3(256), 0, s, w, tab, g, member, sp);
@@ -271,7 +307,9 @@ int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const Disp
     hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, rank, sp);
     return (int)hipGetLastError();
   }
-#define PPLX_ROW_KERNEL_ARGS rank, sp
+  const uint64_t row_bytes = (uint64_t)w.G * w.M * w.K * (w.Hb + 4ull * w.S);
+  const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
+#define PPLX_ROW_KERNEL_ARGS rank, sp, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(split_unpack);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT

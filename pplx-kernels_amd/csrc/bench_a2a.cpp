@@ -3,10 +3,17 @@
 // combine as one call (send+recv) and split into send and recv, HIP events on the stream,
 // 10 samples per repeat after warm-up, mean and standard deviation, and the payload
 // bandwidth by the reference's formula (tokens * K * bytes per token, :266-275) summed over
-// the simulated ranks.  All ranks run in this process on one GPU.
+// the simulated ranks.  The phases run in the reference's order (:183-203)
+//     dispatch, combine, dispatch SEND, gap, dispatch RECV, combine SEND, gap, combine RECV
+// where the gap is a kernel that sleeps for 100 us in place of the experts' compute.  A last
+// section runs a SEND phase on one stream while the gap kernel occupies another, to show that
+// a split phase overlaps with independent work.  All ranks run in this process on one GPU.
 //
-//   bench_a2a [ranks=8] [repeats=10]
+//   bench_a2a [ranks=8] [repeats=10] [quick]
+#include <hip/hip_runtime.h>
+
 #include <cmath>
+#include <string>
 
 #include "harness.h"
 
@@ -17,6 +24,24 @@ namespace {
 struct Config {
   uint32_t tokens, experts, k, hidden;
 };
+
+// Stands in for the experts' compute between the phases (the reference's sleepOnStream over
+// csrc/core/kernels.cu:8-12): one wavefront that naps until `us` microseconds of the 100 MHz
+// wall clock have passed, in at most `max_naps` naps, so that it ends whatever the clock does.
+__global__ void gap_kernel(uint32_t us, uint32_t max_naps) {
+  const uint64_t start = wall_clock64();
+  for (uint32_t i = 0; i < max_naps; ++i) {
+    if (wall_clock64() - start >= (uint64_t)us * 100u) break;
+    __builtin_amdgcn_s_sleep(32);
+  }
+}
+
+constexpr uint32_t kGapUs = 100;
+
+void gap(hipStream_t stream) {
+  hipLaunchKernelGGL(gap_kernel, dim3(1), dim3(64), 0, stream, kGapUs, 4 * kGapUs);
+  HIP_OK(hipGetLastError());
+}
 
 struct Stat {
   double mean, stddev;
@@ -61,6 +86,7 @@ World make_world(const Config &cfg, uint32_t R, bool fp8) {
   c.hidden_dim_bytes = w.Hb;
   c.hidden_dim_scale_bytes = w.scale_dim * 4;
   A2A_OK(pplx_a2a_world_create(&c, 0, &w.world));
+  A2A_OK(pplx_a2a_world_reserve_split(w.world, 2));  // bf16 expert_y
   w.ranks.resize(R);
   std::mt19937 gen(1234);
   for (uint32_t r = 0; r < R; ++r) {
@@ -142,8 +168,10 @@ void bench_config(const Config &cfg, uint32_t R, bool fp8, unsigned repeats, hip
       timed([&] { dispatch(PPLX_A2A_SPLIT_NONE); });
       timed([&] { combine(PPLX_A2A_SPLIT_NONE); });
       timed([&] { dispatch(PPLX_A2A_SPLIT_SEND); });
+      gap(stream);
       timed([&] { dispatch(PPLX_A2A_SPLIT_RECV); });
       timed([&] { combine(PPLX_A2A_SPLIT_SEND); });
+      gap(stream);
       timed([&] { combine(PPLX_A2A_SPLIT_RECV); });
     }
     HIP_OK(hipStreamSynchronize(stream));
@@ -167,8 +195,57 @@ void bench_config(const Config &cfg, uint32_t R, bool fp8, unsigned repeats, hip
          s[3].mean, s[3].stddev, pairs * bytes_per_token / s[0].mean * 1e-3, s[1].mean, s[1].stddev,
          s[4].mean, s[4].stddev, s[5].mean, s[5].stddev, pairs * w.H * 2.0 / s[1].mean * 1e-3);
   fflush(stdout);
+  if (cfg.tokens == 128 && cfg.experts == 256) {
+    printf("     send+recv against one call: dispatch %.2fx, combine %.2fx\n",
+           (s[2].mean + s[3].mean) / s[0].mean, (s[4].mean + s[5].mean) / s[1].mean);
+  }
   for (auto &row : ev)
     for (auto &e : row) HIP_OK(hipEventDestroy(e));
+  free_world(w);
+}
+
+// dispatch SEND on one stream while the gap kernel (the "experts") runs on another: the pair
+// takes about as long as the longer of the two when the phases overlap, their sum when not.
+void bench_overlap(const Config &cfg, uint32_t R, hipStream_t comm) {
+  World w = make_world(cfg, R, true);
+  hipStream_t compute;
+  HIP_OK(hipStreamCreate(&compute));
+  hipEvent_t begin, end, fork, join;
+  for (hipEvent_t *e : {&begin, &end, &fork, &join}) HIP_OK(hipEventCreate(e));
+  auto send = [&] {
+    for (uint32_t r = 0; r < R; ++r) A2A_OK(pplx_a2a_dispatch(w.ranks[r], &w.d[r], PPLX_A2A_SPLIT_SEND, comm));
+  };
+  auto recv = [&] {
+    for (uint32_t r = 0; r < R; ++r) A2A_OK(pplx_a2a_dispatch(w.ranks[r], &w.d[r], PPLX_A2A_SPLIT_RECV, comm));
+  };
+  auto measure = [&](bool with_send, bool with_gap) {
+    double total = 0;
+    const int reps = 20;
+    for (int i = -3; i < reps; ++i) {
+      HIP_OK(hipEventRecord(begin, comm));
+      if (with_gap) {
+        HIP_OK(hipEventRecord(fork, comm));
+        HIP_OK(hipStreamWaitEvent(compute, fork, 0));
+        gap(compute);
+        HIP_OK(hipEventRecord(join, compute));
+      }
+      if (with_send) send();
+      if (with_gap) HIP_OK(hipStreamWaitEvent(comm, join, 0));
+      HIP_OK(hipEventRecord(end, comm));
+      if (with_send) recv();  // completes the step
+      HIP_OK(hipStreamSynchronize(comm));
+      float ms = 0;
+      HIP_OK(hipEventElapsedTime(&ms, begin, end));
+      if (i >= 0) total += ms * 1e3;
+    }
+    return total / reps;
+  };
+  const double t_send = measure(true, false), t_gap = measure(false, true), t_both = measure(true, true);
+  printf("overlap, %u tok x %u ranks: dispatch SEND alone %.1f us, gap kernel alone %.1f us, "
+         "SEND on one stream with the gap kernel on another %.1f us (sum %.1f)\n",
+         cfg.tokens, R, t_send, t_gap, t_both, t_send + t_gap);
+  for (hipEvent_t e : {begin, end, fork, join}) HIP_OK(hipEventDestroy(e));
+  HIP_OK(hipStreamDestroy(compute));
   free_world(w);
 }
 
@@ -177,6 +254,7 @@ void bench_config(const Config &cfg, uint32_t R, bool fp8, unsigned repeats, hip
 int main(int argc, char **argv) {
   const uint32_t R = argc > 1 ? (uint32_t)atoi(argv[1]) : 8;
   const unsigned repeats = argc > 2 ? (unsigned)atoi(argv[2]) : 10;
+  const bool quick = argc > 3 && std::string(argv[3]) == "quick";
   int n_dev = 0;
   if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
     fprintf(stderr, "bench_a2a: no GPU visible\n");
@@ -188,6 +266,7 @@ int main(int argc, char **argv) {
   std::vector<Config> configs = {{1, 8, 4, 128}, {4, 8, 6, 2048}};
   for (uint32_t experts : {8u, 16u, 64u, 256u})
     for (uint32_t tokens : {1u, 4u, 16u, 64u, 128u}) configs.push_back({tokens, experts, 8, 7168});
+  if (quick) configs = {{4, 8, 6, 2048}, {128, 256, 8, 7168}};
   for (bool fp8 : {true, false}) {
     printf("%s rows, %u simulated ranks on one GPU, times in us (host-launched, per-rank calls)\n",
            fp8 ? "FP8 + block scales" : "BF16", R);
@@ -198,6 +277,7 @@ int main(int argc, char **argv) {
       bench_config(cfg, R, fp8, repeats, stream);
     }
   }
+  if (256 % R == 0) bench_overlap({128, 256, 8, 7168}, R, stream);
   HIP_OK(hipStreamDestroy(stream));
   return 0;
 }

@@ -165,6 +165,15 @@ bool run_case(const Geometry &geo, Mode mode, hipStream_t stream) {
       A2A_OK(pplx_a2a_dispatch(ranks[r], &a, PPLX_A2A_SPLIT_NONE, stream));
     }
   } else {
+    // dispatch / combine never allocate: a split call on a world without staging is refused
+    {
+      auto a = dispatch_args(0);
+      if (pplx_a2a_dispatch(ranks[0], &a, PPLX_A2A_SPLIT_SEND, stream) != PPLX_A2A_INVALID_STATE) {
+        printf("  FAIL %s [%s]: split call accepted without reserved staging\n", geo.name, mode_name(mode));
+        return false;
+      }
+      A2A_OK(pplx_a2a_world_reserve_split(world, y_dtype == PPLX_A2A_F32 ? 4 : 2));
+    }
     for (uint32_t r = 0; r < geo.R; ++r) {
       auto a = dispatch_args(r);
       A2A_OK(pplx_a2a_dispatch(ranks[r], &a, PPLX_A2A_SPLIT_SEND, stream));

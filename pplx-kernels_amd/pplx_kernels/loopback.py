@@ -194,7 +194,8 @@ class LoopbackWorld:
     def faults(self) -> int:
         """Sticky device-side fault bits since the last call (synchronises the stream):
         1 = a routed row did not fit ``out_expert_x.size(1)``, 2 = an expert index was out of
-        range, 4 = combine met a slot beyond ``expert_y.size(1)``."""
+        range, 4 = combine met a slot beyond ``expert_y.size(1)``, 8 = an expert id repeated
+        inside one token was dropped, 16 = a ``bound_m`` beyond ``max_num_tokens`` was clamped."""
         bits = ctypes.c_uint32()
         stream = torch.cuda.current_stream().cuda_stream
         ops.check_status(

@@ -49,6 +49,7 @@ EXPORTED_SYMBOLS = (
     "pplx_a2a_combine",
     "pplx_a2a_world_dispatch",
     "pplx_a2a_world_combine",
+    "pplx_a2a_world_reserve_split",
     "pplx_a2a_world_faults",
     "pplx_a2a_graph_begin_capture",
     "pplx_a2a_graph_end_capture",
@@ -56,6 +57,7 @@ EXPORTED_SYMBOLS = (
     "pplx_a2a_graph_destroy",
     "pplx_a2a_last_error",
     "pplx_a2a_version",
+    "pplx_a2a_build_id",
 )
 
 
@@ -153,6 +155,7 @@ def load_library() -> ctypes.CDLL:
         lib.pplx_a2a_combine.argtypes = [vp, ctypes.POINTER(CombineArgs), i32, vp]
         lib.pplx_a2a_world_dispatch.argtypes = [vp, ctypes.POINTER(DispatchArgs), vp]
         lib.pplx_a2a_world_combine.argtypes = [vp, ctypes.POINTER(CombineArgs), vp]
+        lib.pplx_a2a_world_reserve_split.argtypes = [vp, u32]
         lib.pplx_a2a_world_faults.argtypes = [vp, vp, ctypes.POINTER(u32)]
         lib.pplx_a2a_graph_begin_capture.argtypes = [vp]
         lib.pplx_a2a_graph_end_capture.argtypes = [vp, ctypes.POINTER(vp)]
@@ -160,6 +163,7 @@ def load_library() -> ctypes.CDLL:
         lib.pplx_a2a_graph_destroy.argtypes = [vp]
         lib.pplx_a2a_last_error.restype = ctypes.c_char_p
         lib.pplx_a2a_version.restype = ctypes.c_char_p
+        lib.pplx_a2a_build_id.restype = ctypes.c_char_p
         for name in EXPORTED_SYMBOLS:
             getattr(lib, name)  # AttributeError here means a stale or foreign library
         _lib = lib
@@ -190,6 +194,9 @@ class _World:
         # ranks that called earlier are kept alive until then: a temporary such as
         # ``x.to(device)`` must not go back to the caching allocator before it is read.
         self.pending: dict[str, dict[int, tuple]] = {"dispatch": {}, "combine": {}}
+        # Widest expert_y element (bytes) that split-mode staging has been reserved for;
+        # -1 = none reserved yet.
+        self.split_reserved = -1
 
     def hold(self, kind: str, fptr: int, tensors: tuple) -> None:
         held = self.pending[kind]
@@ -299,6 +306,18 @@ def _destroy_all() -> None:
 
 
 atexit.register(_destroy_all)
+
+
+def reserve_split(world: _World, expert_y_elem_bytes: int) -> None:
+    """Split send / recv calls go through staging that the library never allocates inside
+    dispatch / combine.  The reference's callers do not know of it, so the binding reserves it
+    the first time a rank splits a call (and widens it for a wider ``expert_y`` dtype); like
+    any allocation this synchronises and cannot happen under stream capture: run one eager
+    step before capturing split calls, or call this up front."""
+    if world.split_reserved >= expert_y_elem_bytes:
+        return
+    check_status(load_library().pplx_a2a_world_reserve_split(world.ptr, expert_y_elem_bytes))
+    world.split_reserved = expert_y_elem_bytes
 
 
 def is_live(fptr: int) -> bool:
@@ -525,6 +544,8 @@ def _dispatch(
         dp_x_scale, indices, bound_m,
     )  # fmt: skip
     mode = split_mode(do_send, do_recv)
+    if mode != SPLIT_NONE:
+        reserve_split(world, 0)
     # The library selects the world's device for the launch and restores the caller's; the
     # stream is the current one of the tensors' device (csrc/bindings/all_to_all_ops.cpp:163,194).
     check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
@@ -552,6 +573,8 @@ def _combine(
         raise RuntimeError("pplx_kernels: invalid state: the handle has been destroyed")
     args = pack_combine_args(out_tokens, indices, weights, expert_y, bound_m)
     mode = split_mode(do_send, do_recv)
+    if mode != SPLIT_NONE:
+        reserve_split(world, expert_y.element_size())
     check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
     if mode == SPLIT_NONE:
         world.hold("combine", fptr, (out_tokens, indices, weights, expert_y, bound_m))

@@ -27,11 +27,32 @@ def declared_symbols() -> list[str]:
 def test_library_exports_every_declared_symbol():
     lib = ops.load_library()
     names = declared_symbols()
-    assert len(names) >= 17
+    assert len(names) >= 19
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in include/pplx_a2a.h but not exported"
     assert sorted(ops.EXPORTED_SYMBOLS) == names
     assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.pplx_a2a_version())
+
+
+def test_library_is_built_from_the_sources_in_the_tree():
+    """The library reports a hash of the sources it was built from; a kernel edit without a
+    rebuild (tests load what is built, they do not build) shows up here."""
+    import glob
+    import hashlib
+
+    csrc = os.path.join(ROOT, "pplx-kernels_amd", "csrc")
+    files = sorted(
+        os.path.basename(p)
+        for pat in ("*.hip", "a2a_*.h", "a2a_capi.cpp")
+        for p in glob.glob(os.path.join(csrc, pat))
+    )
+    h = hashlib.sha256()
+    for name in files:
+        h.update(open(os.path.join(csrc, name), "rb").read())
+    h.update(open(HEADER, "rb").read())
+    assert ops.load_library().pplx_a2a_build_id().decode() == h.hexdigest()[:16], (
+        "libpplx_kernels.so is stale: run `make -C pplx-kernels_amd/csrc`"
+    )
 
 
 def test_ctypes_structs_match_the_header_layout():
@@ -94,6 +115,7 @@ def test_null_arguments_are_status_codes_not_crashes():
     assert lib.pplx_a2a_combine(None, None, 0, None) == 1
     assert lib.pplx_a2a_world_dispatch(None, None, None) == 1
     assert lib.pplx_a2a_world_faults(None, None, None) == 1
+    assert lib.pplx_a2a_world_reserve_split(None, 2) == 1
     assert lib.pplx_a2a_graph_launch(None, None) == 1
     assert lib.pplx_a2a_destroy(None) == 0 and lib.pplx_a2a_world_destroy(None) == 0
     assert lib.pplx_a2a_graph_destroy(None) == 0
