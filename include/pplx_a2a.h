@@ -182,6 +182,29 @@ int pplx_a2a_world_dispatch(pplx_a2a_world_t *world, const pplx_a2a_dispatch_arg
 int pplx_a2a_world_combine(pplx_a2a_world_t *world, const pplx_a2a_combine_args_t *per_rank,
                            void *stream);
 
+/* One step (dispatch, combine, or dispatch then combine) for all ranks without a
+ * world and without any allocation.  It has no counterpart in the reference; it
+ * is for callers that cannot allocate device memory around the call: code under
+ * hipGraph capture that has no world yet, tight serving loops, harnesses that
+ * forbid hipMalloc.  `dispatch_per_rank` / `combine_per_rank` are host arrays
+ * of world_size entries as for pplx_a2a_world_dispatch / _combine (either may be
+ * NULL to skip that half); the kernels and the results are the same.  The state
+ * a world would own (slot map, routing tile counts) lives in a 4 MiB array that
+ * is part of the library's code object on every GPU; a geometry that needs more
+ * (world_size / dp_size * max_num_tokens * experts_per_token * 4 bytes of slot
+ * map plus the tile counts), or more than 64 ranks, is refused with
+ * PPLX_A2A_INVALID_ARGUMENT / PPLX_A2A_UNSUPPORTED.  The slot map written by a
+ * dispatch stays there for the combine of a later call.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU (different streams or
+ * threads) race, and a step of a different geometry overwrites the slot map.
+ * `fault_bits`: optional device word that the kernels OR the fault bits of
+ * pplx_a2a_world_faults into (the caller clears and reads it); NULL discards them.
+ * Calls no hipMalloc / hipFree and never synchronises. */
+int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
+                         const pplx_a2a_dispatch_args_t *dispatch_per_rank,
+                         const pplx_a2a_combine_args_t *combine_per_rank, uint32_t *fault_bits,
+                         void *stream);
+
 /* Allocates the staging that split send / recv calls go through (the reference
  * allocates its inboxes in the constructor, csrc/all_to_all/intranode.cpp:37-136;
  * here a world that never splits does not pay for them): about

@@ -180,9 +180,32 @@ int check_config(const pplx_a2a_config_t &c) {
   return PPLX_A2A_OK;
 }
 
-int convert_dispatch(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_dispatch_args_t &a,
+// The geometry part of a WorldDev (everything but the pointers) for a checked configuration.
+void fill_geometry(const pplx_a2a_config_t &cfg, WorldDev &d) {
+  d.R = cfg.world_size;
+  d.dp = cfg.dp_size;
+  d.G = d.R / d.dp;
+  d.M = (uint32_t)cfg.max_num_tokens;
+  d.E = (uint32_t)cfg.num_experts;
+  d.L = d.E / d.R;
+  d.K = (uint32_t)cfg.experts_per_token;
+  d.H = (uint32_t)cfg.hidden_dim;
+  d.Hb = (uint32_t)cfg.hidden_dim_bytes;
+  d.S = (uint32_t)(cfg.hidden_dim_scale_bytes / 4);
+  // Routing tiles of a whole step: small enough that a step has a few hundred of them (a tile
+  // is one workgroup, and routing is a chain of short launches that only parallelism shortens),
+  // at most 16 chunks of 64 tokens, and such that the LDS tables fit 64 KiB.
+  const uint64_t step_chunks = ((uint64_t)d.G * d.M + kWave - 1) / kWave;
+  d.tile_chunks = 1;
+  while (d.tile_chunks < 16 && step_chunks / d.tile_chunks > 256) d.tile_chunks *= 2;
+  while (d.tile_chunks > 1 && route_lds_bytes(d.E, d.tile_chunks) > 65536u) d.tile_chunks /= 2;
+  const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
+  d.num_tiles = (uint32_t)(((uint64_t)d.G * d.M + tile_tokens - 1) / tile_tokens);
+}
+
+int convert_dispatch(const WorldDev &geo, uint32_t rank, const pplx_a2a_dispatch_args_t &a,
                      DispatchRank *out) {
-  const uint32_t S = w.dev.S;
+  const uint32_t S = geo.S;
   if (!a.out_expert_num_tokens)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_num_tokens is NULL", rank);
   if (!a.out_expert_x) return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x is NULL", rank);
@@ -200,9 +223,9 @@ int convert_dispatch(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_disp
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_expert_x_rows is negative", rank);
   // csrc/all_to_all/intranode_dispatch.cu:65 asserts numSendTokens <= maxNumTokens; a device-side
   // bound_m beyond the limit is clamped and reported through the fault word instead.
-  if (!a.bound_m && a.m > w.dev.M)
-    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, w.dev.M);
-  const uint64_t rows = a.out_expert_x_rows ? (uint64_t)a.out_expert_x_rows : (uint64_t)w.dev.M * w.dev.G;
+  if (!a.bound_m && a.m > geo.M)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, geo.M);
+  const uint64_t rows = a.out_expert_x_rows ? (uint64_t)a.out_expert_x_rows : (uint64_t)geo.M * geo.G;
   DispatchRank d{};
   d.out_num_tokens = a.out_expert_num_tokens;
   d.out_num_tokens_stride = a.out_expert_num_tokens_stride;
@@ -228,14 +251,14 @@ int convert_dispatch(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_disp
 
 size_t dtype_size(int dt) { return dt == PPLX_A2A_F32 ? 4 : 2; }
 
-int convert_combine(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_combine_args_t &a,
+int convert_combine(const WorldDev &geo, uint32_t rank, const pplx_a2a_combine_args_t &a,
                     CombineRank *out) {
   // csrc/bindings/all_to_all_ops.cpp:265-310
   if (a.in_dtype != PPLX_A2A_F32 && a.in_dtype != PPLX_A2A_BF16 && a.in_dtype != PPLX_A2A_F16)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Unsupported dtype for expertY");
   if (a.out_dtype != PPLX_A2A_BF16 && a.out_dtype != PPLX_A2A_F16)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Unsupported dtype for outTokens");
-  if (w.dev.H % 8 != 0)
+  if (geo.H % 8 != 0)
     return fail(PPLX_A2A_UNSUPPORTED, "combine needs hidden_dim to be a multiple of 8");
   if (!a.expert_y) return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y is NULL", rank);
   if (a.m > 0 && (!a.out_tokens || !a.indices || !a.weights))
@@ -248,9 +271,9 @@ int convert_combine(const pplx_a2a_world &w, uint32_t rank, const pplx_a2a_combi
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: out_tokens must be 16-byte aligned with a 16-byte row stride", rank);
   if (a.expert_y_rows < 0)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: expert_y_rows is negative", rank);
-  if (!a.bound_m && a.m > w.dev.M)
-    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, w.dev.M);
-  const uint64_t rows = a.expert_y_rows ? (uint64_t)a.expert_y_rows : (uint64_t)w.dev.M * w.dev.G;
+  if (!a.bound_m && a.m > geo.M)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "rank %u: %u tokens exceed max_num_tokens %u", rank, a.m, geo.M);
+  const uint64_t rows = a.expert_y_rows ? (uint64_t)a.expert_y_rows : (uint64_t)geo.M * geo.G;
   CombineRank c{};
   c.out_tokens = a.out_tokens;
   c.out_stride_row = a.out_tokens_stride_row;
@@ -323,22 +346,23 @@ uint32_t pick_vector_for(uint32_t K, const uint32_t *indices, uint32_t at_most =
 }
 
 // ... that suits the indices of every rank of the pending step.
-uint32_t pick_vector_of(const pplx_a2a_world &w) {
+uint32_t pick_vector_of(const WorldDev &d, const DispatchRank *rows) {
   uint32_t pv = 4;
-  for (const DispatchRank &r : w.pend_dispatch) pv = pick_vector_for(w.dev.K, r.indices, pv);
+  for (uint32_t r = 0; r < d.R; ++r) pv = pick_vector_for(d.K, rows[r].indices, pv);
   return pv;
 }
+uint32_t pick_vector_of(const pplx_a2a_world &w) { return pick_vector_of(w.dev, w.pend_dispatch.data()); }
 
 // The members of a DP group hold the same tokens (csrc/all_to_all/intranode_dispatch.cu:97
 // strides one token list over them), so they must agree on how many rows there are: the
 // kernels take the count from the group's first member and read every member's rows.
-int check_groups(const pplx_a2a_world &w) {
-  const uint32_t dp = w.dev.dp;
+int check_groups(const WorldDev &d, const DispatchRank *rows) {
+  const uint32_t dp = d.dp;
   if (dp == 1) return PPLX_A2A_OK;
-  for (uint32_t g = 0; g < w.dev.G; ++g) {
-    const DispatchRank &head = w.pend_dispatch[g * dp];
+  for (uint32_t g = 0; g < d.G; ++g) {
+    const DispatchRank &head = rows[g * dp];
     for (uint32_t i = 1; i < dp; ++i) {
-      const DispatchRank &member = w.pend_dispatch[g * dp + i];
+      const DispatchRank &member = rows[g * dp + i];
       if (member.m != head.m || (member.bound_m == nullptr) != (head.bound_m == nullptr))
         return fail(PPLX_A2A_INVALID_ARGUMENT,
                     "ranks %u and %u share a DP group but pass %u and %u tokens (or only one of them a bound_m)",
@@ -389,7 +413,7 @@ int run_ordered(pplx_a2a_world &w, const std::vector<void *> &streams, void *lau
 }
 
 int run_dispatch(pplx_a2a_world &w, void *stream) {
-  int st = check_groups(w);
+  int st = check_groups(w.dev, w.pend_dispatch.data());
   if (st) return st;
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
@@ -641,30 +665,18 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
   DeviceScope scope(device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", device);
 
+  {
+    // The first world on a device also looks up that device's copy of the library's static
+    // scratch array, so that pplx_a2a_static_step finds it ready.
+    void *unused = nullptr;
+    LAUNCH_TRY(static_scratch_address(device, &unused));
+  }
   pplx_a2a_world *w = new (std::nothrow) pplx_a2a_world();
   if (!w) return fail(PPLX_A2A_HIP_ERROR, "out of host memory");
   w->cfg = *cfg;
   w->device = device;
   WorldDev &d = w->dev;
-  d.R = cfg->world_size;
-  d.dp = cfg->dp_size;
-  d.G = d.R / d.dp;
-  d.M = (uint32_t)cfg->max_num_tokens;
-  d.E = (uint32_t)cfg->num_experts;
-  d.L = d.E / d.R;
-  d.K = (uint32_t)cfg->experts_per_token;
-  d.H = (uint32_t)cfg->hidden_dim;
-  d.Hb = (uint32_t)cfg->hidden_dim_bytes;
-  d.S = (uint32_t)(cfg->hidden_dim_scale_bytes / 4);
-  // Routing tiles of a whole step: small enough that a step has a few hundred of them (a tile
-  // is one workgroup, and routing is a chain of short launches that only parallelism shortens),
-  // at most 16 chunks of 64 tokens, and such that the LDS tables fit 64 KiB.
-  const uint64_t step_chunks = ((uint64_t)d.G * d.M + kWave - 1) / kWave;
-  d.tile_chunks = 1;
-  while (d.tile_chunks < 16 && step_chunks / d.tile_chunks > 256) d.tile_chunks *= 2;
-  while (d.tile_chunks > 1 && route_lds_bytes(d.E, d.tile_chunks) > 65536u) d.tile_chunks /= 2;
-  const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
-  d.num_tiles = (uint32_t)(((uint64_t)d.G * d.M + tile_tokens - 1) / tile_tokens);
+  fill_geometry(*cfg, d);
 
   auto cleanup = [&]() {
     for (hipEvent_t ev : w->rank_events) (void)hipEventDestroy(ev);
@@ -781,7 +793,7 @@ int pplx_a2a_dispatch(pplx_a2a_t *h, const pplx_a2a_dispatch_args_t *args, int s
       split_mode != PPLX_A2A_SPLIT_RECV)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
   DispatchRank row;
-  int st = convert_dispatch(w, h->rank, *args, &row);
+  int st = convert_dispatch(w.dev, h->rank, *args, &row);
   if (st) return st;
   std::lock_guard<std::mutex> lock(w.mu);
   if (split_mode != PPLX_A2A_SPLIT_NONE) return split_dispatch(w, h->rank, row, split_mode, stream);
@@ -806,7 +818,7 @@ int pplx_a2a_combine(pplx_a2a_t *h, const pplx_a2a_combine_args_t *args, int spl
       split_mode != PPLX_A2A_SPLIT_RECV)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "Invalid split mode");
   CombineRank row;
-  int st = convert_combine(w, h->rank, *args, &row);
+  int st = convert_combine(w.dev, h->rank, *args, &row);
   if (st) return st;
   std::lock_guard<std::mutex> lock(w.mu);
   if (split_mode != PPLX_A2A_SPLIT_NONE)
@@ -839,7 +851,7 @@ int pplx_a2a_world_dispatch(pplx_a2a_world_t *w, const pplx_a2a_dispatch_args_t 
   if (w->n_arrived_dispatch != 0 || w->n_dsend != 0 || w->n_drecv != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a per-rank dispatch step is still being assembled");
   for (uint32_t r = 0; r < w->dev.R; ++r) {
-    int st = convert_dispatch(*w, r, per_rank[r], &w->pend_dispatch[r]);
+    int st = convert_dispatch(w->dev, r, per_rank[r], &w->pend_dispatch[r]);
     if (st) return st;
   }
   return run_dispatch(*w, stream);
@@ -854,7 +866,7 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *w, const pplx_a2a_combine_args_t *p
   for (uint32_t r = 0; r < w->dev.R; ++r) {
     if (per_rank[r].in_dtype != per_rank[0].in_dtype || per_rank[r].out_dtype != per_rank[0].out_dtype)
       return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
-    int st = convert_combine(*w, r, per_rank[r], &w->pend_combine[r]);
+    int st = convert_combine(w->dev, r, per_rank[r], &w->pend_combine[r]);
     if (st) return st;
   }
   w->combine_in_dtype = per_rank[0].in_dtype;
@@ -866,6 +878,69 @@ int pplx_a2a_world_reserve_split(pplx_a2a_world_t *w, uint32_t expert_y_elem_byt
   if (!w) return fail(PPLX_A2A_INVALID_ARGUMENT, "world is NULL");
   std::lock_guard<std::mutex> lock(w->mu);
   return reserve_split(*w, expert_y_elem_bytes);
+}
+
+int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
+                         const pplx_a2a_dispatch_args_t *dispatch_per_rank,
+                         const pplx_a2a_combine_args_t *combine_per_rank, uint32_t *fault_bits,
+                         void *stream) {
+  if (!cfg) return fail(PPLX_A2A_INVALID_ARGUMENT, "cfg is NULL");
+  if (!dispatch_per_rank && !combine_per_rank)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "neither a dispatch nor a combine to run");
+  int st = check_config(*cfg);
+  if (st) return st;
+  if (cfg->world_size > kInlineRanks)
+    return fail(PPLX_A2A_UNSUPPORTED, "the static step serves worlds of up to %u ranks, not %u", kInlineRanks,
+                cfg->world_size);
+  WorldDev d{};
+  fill_geometry(*cfg, d);
+  // Scratch layout: the fault word, the slot map (the hand-off from dispatch to combine, kept
+  // from one call to the next), the routing tiles' counts.
+  const size_t slot_bytes = sizeof(uint32_t) * (size_t)d.G * d.M * d.K;
+  const size_t tile_bytes = sizeof(uint32_t) * (size_t)d.num_tiles * d.E;
+  const size_t slot_at = 256, tile_at = slot_at + (slot_bytes + 255) / 256 * 256;
+  const size_t needed = tile_at + tile_bytes;
+  if (needed > kStaticScratchBytes)
+    return fail(PPLX_A2A_INVALID_ARGUMENT,
+                "the geometry needs %zu bytes of scratch, the library's static array holds %zu: "
+                "use a world (pplx_a2a_world_create) for it", needed, (size_t)kStaticScratchBytes);
+  int n_dev = 0;
+  HIP_TRY(hipGetDeviceCount(&n_dev));
+  if (device < 0 || device >= n_dev)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "device %d out of range (%d visible)", device, n_dev);
+  DeviceScope scope(device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", device);
+  void *base = nullptr;
+  LAUNCH_TRY(static_scratch_address(device, &base));
+  uint8_t *scratch = static_cast<uint8_t *>(base);
+  d.faults = fault_bits ? fault_bits : reinterpret_cast<uint32_t *>(scratch);
+  d.slot_map = reinterpret_cast<uint32_t *>(scratch + slot_at);
+  d.tile_cnt = reinterpret_cast<uint32_t *>(scratch + tile_at);
+
+  if (dispatch_per_rank) {
+    DispatchRank rows[kInlineRanks];
+    for (uint32_t r = 0; r < d.R; ++r) {
+      st = convert_dispatch(d, r, dispatch_per_rank[r], &rows[r]);
+      if (st) return st;
+    }
+    st = check_groups(d, rows);
+    if (st) return st;
+    ProfilerRange range("dispatch");
+    LAUNCH_TRY(launch_dispatch(d, rows, pick_vector_of(d, rows), stream));
+  }
+  if (combine_per_rank) {
+    CombineRank rows[kInlineRanks];
+    for (uint32_t r = 0; r < d.R; ++r) {
+      if (combine_per_rank[r].in_dtype != combine_per_rank[0].in_dtype ||
+          combine_per_rank[r].out_dtype != combine_per_rank[0].out_dtype)
+        return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
+      st = convert_combine(d, r, combine_per_rank[r], &rows[r]);
+      if (st) return st;
+    }
+    ProfilerRange range("combine");
+    LAUNCH_TRY(launch_combine(d, rows, combine_per_rank[0].in_dtype, combine_per_rank[0].out_dtype, stream));
+  }
+  return PPLX_A2A_OK;
 }
 
 int pplx_a2a_world_faults(pplx_a2a_world_t *w, void *stream, uint32_t *out_bits) {

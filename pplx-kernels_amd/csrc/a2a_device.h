@@ -7,6 +7,7 @@
 // csrc/all_to_all/intranode_combine.cu:16-47.
 #pragma once
 
+#include <cstddef>
 #include <cstdint>
 
 namespace pplx_amd {
@@ -130,6 +131,12 @@ constexpr uint32_t kFusedMaxTokens = 16384;
 // A fused launch whose rows (all picks of all tokens) stay within this many bytes stores them
 // write-through into the 256 MB last-level cache instead of streaming them past it.
 constexpr uint64_t kWriteThroughMaxBytes = 128ull << 20;
+
+// Device memory that pplx_a2a_static_step works in instead of a world's allocations: a fixed
+// array inside the library's code object (a2a_static.hip), one copy per GPU.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+// Address of the calling thread's current device's copy (looked up once per device).
+int static_scratch_address(int device, void **out);
 
 struct BindDispatchBatch {
   uint32_t first, count;

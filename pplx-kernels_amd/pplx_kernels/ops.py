@@ -49,6 +49,7 @@ EXPORTED_SYMBOLS = (
     "pplx_a2a_combine",
     "pplx_a2a_world_dispatch",
     "pplx_a2a_world_combine",
+    "pplx_a2a_static_step",
     "pplx_a2a_world_reserve_split",
     "pplx_a2a_world_faults",
     "pplx_a2a_graph_begin_capture",
@@ -155,6 +156,9 @@ def load_library() -> ctypes.CDLL:
         lib.pplx_a2a_combine.argtypes = [vp, ctypes.POINTER(CombineArgs), i32, vp]
         lib.pplx_a2a_world_dispatch.argtypes = [vp, ctypes.POINTER(DispatchArgs), vp]
         lib.pplx_a2a_world_combine.argtypes = [vp, ctypes.POINTER(CombineArgs), vp]
+        lib.pplx_a2a_static_step.argtypes = [
+            ctypes.POINTER(Config), i32, ctypes.POINTER(DispatchArgs), ctypes.POINTER(CombineArgs), vp, vp,
+        ]  # fmt: skip
         lib.pplx_a2a_world_reserve_split.argtypes = [vp, u32]
         lib.pplx_a2a_world_faults.argtypes = [vp, vp, ctypes.POINTER(u32)]
         lib.pplx_a2a_graph_begin_capture.argtypes = [vp]
