@@ -1,18 +1,23 @@
 """Benchmark of the MoE dispatch + combine hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--only] [--no-cpu]
 
-A *step* is one dispatch + one combine over all simulated ranks of the workload, replayed
-from a captured hipGraph (inputs resident in HBM).  To keep the working set from living in
-the 256 MB last-level cache between steps, the steps rotate over several independent buffer
-sets, so every timed step touches memory that was last used several steps ago.
+A *step* is one dispatch + one combine over all simulated ranks of a workload, inputs resident
+in HBM.  To keep the working set from living in the 256 MB last-level cache between steps, the
+steps rotate over several independent buffer sets, so every timed step touches memory that was
+last used several steps ago.
 
-Prints ONE JSON line.  ``value`` is the mean step latency in microseconds on the workload
-the metric is quoted on (C2: DeepSeek-V3 shape, 128 tokens/rank, 8 simulated ranks).
-``roofline`` is for the dominant kernel (``combine_gather``): algorithmic bytes per launch
-divided by its mean duration, measured with HIP events around graph replays that contain
-only launches of that kernel.  ``cpu_baseline`` times the oracle's vectorised torch CPU port
-of the same step on this host's cores.
+Prints ONE JSON line.  ``value`` is the mean step latency in microseconds on the workload the
+metric is quoted on (C2: DeepSeek-V3 shape, 128 tokens/rank, 8 simulated ranks).  How a step is
+launched is fixed by rule, not picked per run: eager launches of a step whose arguments were
+checked and packed once (``LoopbackWorld.bind``: two library calls per step) for every workload
+but the decode shape C3, which is ONE captured hipGraph replayed 1000 times; the other form is
+reported next to it.  ``workloads`` holds a compact entry for each of C1..C5.
+``roofline`` is for the dominant kernel of the headline workload (``combine_gather``):
+algorithmic bytes per launch divided by its mean duration, measured with HIP events around graph
+replays that contain only launches of that kernel; ``traffic`` is read from the rocprofv3 counter
+summary under ``profiles/``.  ``cpu_baseline`` times the oracle's vectorised torch CPU port of the
+same step on this host's cores.
 """
 
 from __future__ import annotations
@@ -20,6 +25,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -33,14 +39,26 @@ for _p in (os.path.join(ROOT, "pplx-kernels_amd"), ROOT):
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 LLC_BYTES = 256 << 20
-# HBM bytes per combine_gather launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by a copy of known size in the same run (profiles/hbm_traffic_<workload>.txt); counters
-# cannot be read from inside this script, so the figure is carried as a constant per workload.
-MEASURED_COMBINE_TRAFFIC_BYTES = {"C2": 133.0e6, "C5": 4391.9e6}
+GRAPH_REPLAYS_C3 = 1000
+
+
+def measured_traffic_bytes(workload: str, kernel: str):
+    """HBM bytes per launch of `kernel` from profiles/hbm_traffic_<workload>.txt (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size in the same run); None when the
+    summary is not there.  Counters cannot be read from inside this script."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}.txt")
+    try:
+        for line in open(path):
+            fields = line.split()
+            if fields and fields[0] == kernel and re.fullmatch(r"[0-9.]+", fields[-1]):
+                return float(fields[-1]) * 1e6  # last column: total MB
+    except OSError:
+        pass
+    return None
 
 
 def build_steps(spec, groups, cap, n_sets):
-    from tests.all_to_all_utils import DeviceStep
+    from pplx_kernels.workloads import DeviceStep
 
     steps = []
     gen = torch.Generator(device="cuda").manual_seed(7)
@@ -74,6 +92,29 @@ def time_graphs(graphs, order, stream, warmup, repeats=1):
     return start.elapsed_time(end) * 1e3 / (len(order) * repeats)
 
 
+def time_bound(bound, order, stream, warmup, dispatch=True, combine=True):
+    """Mean microseconds per step (or per phase) of eager launches of bound steps, HIP events on
+    the launch stream."""
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def run(i):
+        if dispatch:
+            bound[i].dispatch(stream)
+        if combine:
+            bound[i].combine(stream)
+
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            run(order[i % len(order)])
+        stream.synchronize()
+        start.record(stream)
+        for i in order:
+            run(i)
+        end.record(stream)
+        stream.synchronize()
+    return start.elapsed_time(end) * 1e3 / len(order)
+
+
 def capture(world, stream, body):
     with torch.cuda.stream(stream):
         body()  # eager once: binds tables, warms code objects
@@ -83,8 +124,8 @@ def capture(world, stream, body):
     return cap.graph
 
 
-def measure_workload(name, spec, steps_k, warmup, detail=True):
-    from tests.all_to_all_utils import expert_counts, generate, make_world
+def measure_workload(name, spec, steps_k, warmup):
+    from pplx_kernels.workloads import expert_counts, generate, make_world
 
     groups = generate(spec)
     counts = expert_counts(groups, spec.num_experts)
@@ -92,7 +133,6 @@ def measure_workload(name, spec, steps_k, warmup, detail=True):
     full_cap = spec.max_num_tokens * spec.num_dp_groups
     if spec.num_experts * full_cap * spec.hidden_dim * 3 < (8 << 30):
         cap = full_cap  # small enough: use the reference's own sizing
-    disp_b, comb_b = None, None
     # enough buffer sets that a step's data is evicted before it is used again
     probe_bytes = sum(g.n for g in groups) * spec.experts_per_token * spec.hidden_dim * 3
     n_sets = max(2, min(8, int(2.5 * LLC_BYTES / max(probe_bytes, 1)) + 1))
@@ -103,83 +143,106 @@ def measure_workload(name, spec, steps_k, warmup, detail=True):
     world = make_world(spec, group_name=f"bench-{name}")
     stream = torch.cuda.Stream()
     torch.cuda.synchronize()
+    order = [i % n_sets for i in range(steps_k)]
 
+    # Eager launches of steps packed once (LoopbackWorld.bind): two library calls per step.
+    bound = [st.bind_world(world) for st in steps]
+    bound_us = time_bound(bound, order, stream, warmup)
+    d_us = time_bound(bound, order, stream, warmup, combine=False)
+    c_us = time_bound(bound, order, stream, warmup, dispatch=False)
+
+    # The same step as a captured hipGraph.
     def both(st):
         return lambda: (st.dispatch_world(world), st.combine_world(world))
 
-    step_graphs = [capture(world, stream, both(st)) for st in steps]
-    order = [i % n_sets for i in range(steps_k)]
-    step_us = time_graphs(step_graphs, order, stream, warmup)
+    if name == "C3":
+        # the decode shape: ONE graph, replayed 1000 times back to back
+        graph = capture(world, stream, both(steps[0]))
+        graph_us = time_graphs([graph], [0], stream, warmup, GRAPH_REPLAYS_C3)
+        graph.destroy()
+        graph_note = f"one hipGraph replayed {GRAPH_REPLAYS_C3} times"
+    else:
+        graphs = [capture(world, stream, both(st)) for st in steps]
+        graph_us = time_graphs(graphs, order, stream, warmup)
+        for g in graphs:
+            g.destroy()
+        graph_note = f"{n_sets} hipGraphs (one per buffer set), {len(order)} replays"
+    del bound
 
+    launch_form = "graph_replay" if name == "C3" else "bound_eager"
+    step_us = graph_us if name == "C3" else bound_us
+    pairs = int(sum(g.n for g in groups) * spec.experts_per_token)
     out = {
         "workload": spec.name,
         "tokens": int(sum(g.n for g in groups)),
-        "pairs": int(sum(g.n for g in groups) * spec.experts_per_token),
+        "pairs": pairs,
         "rows_per_expert_capacity": cap,
         "buffer_sets": n_sets,
+        "steps_timed": len(order) if name != "C3" else GRAPH_REPLAYS_C3,
+        "launch_form": launch_form,
+        "step_us": step_us,
+        "bound_eager_step_us": bound_us,
+        "graph_step_us": graph_us,
+        "graph_form": graph_note,
+        "dispatch_us": d_us,
+        "combine_us": c_us,
         "dispatch_bytes": disp_b,
         "combine_bytes": comb_b,
-        "step_us": step_us,
-        "step_GBps": (disp_b + comb_b) / step_us / 1e3,
         "step_hbm_frac": (disp_b + comb_b) / step_us / 1e3 / HBM_PEAK_GBPS,
-    }
-    if detail:
-        d_graphs = [capture(world, stream, lambda st=st: st.dispatch_world(world)) for st in steps]
-        c_graphs = [capture(world, stream, lambda st=st: st.combine_world(world)) for st in steps]
-        reps = max(1, steps_k // n_sets)
-        d_us = time_graphs(d_graphs, list(range(n_sets)), stream, warmup, reps)
-        c_us = time_graphs(c_graphs, list(range(n_sets)), stream, warmup, reps)
-        # eager (host-launched) step for comparison
-        with torch.cuda.stream(stream):
-            for _ in range(3):
-                both(steps[0])()
-            stream.synchronize()
-            t0 = time.perf_counter()
-            for i in range(min(steps_k, 50)):
-                both(steps[i % n_sets])()
-            stream.synchronize()
-            eager_us = (time.perf_counter() - t0) * 1e6 / min(steps_k, 50)
+        "dispatch_hbm_frac": disp_b / d_us / 1e3 / HBM_PEAK_GBPS,
+        "combine_hbm_frac": comb_b / c_us / 1e3 / HBM_PEAK_GBPS,
+        "step_GBps": (disp_b + comb_b) / step_us / 1e3,
         # the reference bench's one-way payload figures (tests/bench_all_to_all.py:131-139):
         # pairs x bytes per dispatched token, pairs x bytes per combined row
-        pairs = out["pairs"]
-        disp_payload = pairs * (spec.hidden_dim_bytes + spec.hidden_dim_scale_bytes)
-        comb_payload = pairs * spec.hidden_dim * spec.out_dtype.itemsize
-        # eager launches of steps packed once (LoopbackWorld.bind): two library calls per step,
-        # same rotating buffer sets, HIP events on the launch stream
-        bound = [st.bind_world(world) for st in steps]
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        with torch.cuda.stream(stream):
-            for i in range(warmup):
-                bound[i % n_sets].dispatch(stream)
-                bound[i % n_sets].combine(stream)
-            stream.synchronize()
-            start.record(stream)
-            for i in order:
-                bound[i].dispatch(stream)
-                bound[i].combine(stream)
-            end.record(stream)
-            stream.synchronize()
-        bound_us = start.elapsed_time(end) * 1e3 / len(order)
-        del bound
-        out.update(
-            bound_eager_step_us=bound_us,
-            dispatch_payload_GBps=disp_payload / d_us / 1e3,
-            combine_payload_GBps=comb_payload / c_us / 1e3,
-            dispatch_us=d_us,
-            combine_us=c_us,
-            dispatch_GBps=disp_b / d_us / 1e3,
-            combine_GBps=comb_b / c_us / 1e3,
-            dispatch_hbm_frac=disp_b / d_us / 1e3 / HBM_PEAK_GBPS,
-            combine_hbm_frac=comb_b / c_us / 1e3 / HBM_PEAK_GBPS,
-            eager_step_us=eager_us,
-        )
-        for g in d_graphs + c_graphs:
-            g.destroy()
-    for g in step_graphs:
-        g.destroy()
+        "dispatch_payload_GBps": pairs * (spec.hidden_dim_bytes + spec.hidden_dim_scale_bytes) / d_us / 1e3,
+        "combine_payload_GBps": pairs * spec.hidden_dim * spec.out_dtype.itemsize / c_us / 1e3,
+    }
     assert world.faults() == 0, "device-side fault bits set during the benchmark"
     world.destroy()
     return out, groups, steps
+
+
+def combine_kernel_roofline(name, spec, steps, comb_b, steps_k):
+    """Roofline of the dominant kernel: graphs holding back-to-back combine_gather launches only,
+    rotating buffer sets; mean launch duration by HIP events on the launch stream."""
+    from pplx_kernels.workloads import make_world
+
+    world = make_world(spec, group_name="bench-roofline")
+    stream = torch.cuda.Stream()
+    n_sets = len(steps)
+    launches_per_graph = 8
+
+    def many_combines(st):
+        def body():
+            for _ in range(launches_per_graph):
+                st.combine_world(world)
+
+        return body
+
+    with torch.cuda.stream(stream):
+        for st in steps:
+            st.dispatch_world(world)  # slot map of this world
+        stream.synchronize()
+    # combine reads the world's slot map, identical for every buffer set (same routing)
+    k_graphs = [capture(world, stream, many_combines(st)) for st in steps]
+    reps = max(1, steps_k // (n_sets * launches_per_graph))
+    per_graph_us = time_graphs(k_graphs, list(range(n_sets)), stream, 2, reps)
+    kernel_us = per_graph_us / launches_per_graph
+    for g in k_graphs:
+        g.destroy()
+    world.destroy()
+    return {
+        "kernel": "combine_gather<bf16,bf16>",
+        "bound": "hbm",
+        "achieved": comb_b / kernel_us / 1e3,
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": comb_b / kernel_us / 1e3 / HBM_PEAK_GBPS,
+        "traffic": measured_traffic_bytes(name, "combine_gather"),
+        "bytes_per_launch": comb_b,
+        "avg_launch_us": kernel_us,
+        "launches_timed": reps * n_sets * launches_per_graph,
+    }
 
 
 def cpu_baseline(spec, groups, budget_s=20.0):
@@ -221,16 +284,27 @@ def cpu_literal_loops(spec):
     import numpy as np
 
     from oracle import a2a_oracle as orc
-    from tests.all_to_all_utils import ORACLE_DTYPE, generate, to_oracle_groups
+    from pplx_kernels.workloads import generate
 
-    og = to_oracle_groups(generate(spec))
+    dtype_code = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+    og = [
+        orc.GroupData(
+            g.x.contiguous().view(torch.uint8).reshape(g.x.shape[0], -1).numpy(),
+            None if g.x_scale is None else g.x_scale.numpy(),
+            g.indices.numpy().astype(np.uint32),
+            g.weights.numpy(),
+            g.n,
+        )
+        for g in generate(spec)
+    ]
     M, E, K, H = spec.max_num_tokens, spec.num_experts, spec.experts_per_token, spec.hidden_dim
     cap = M * spec.num_dp_groups
     rng = np.random.default_rng(1)
-    expert_y = orc.from_float32(rng.standard_normal((E, cap, H), dtype=np.float32), ORACLE_DTYPE[spec.expert_y_dtype])
+    y_dt, out_dt = dtype_code[spec.expert_y_dtype], dtype_code[spec.out_dtype]
+    expert_y = orc.from_float32(rng.standard_normal((E, cap, H), dtype=np.float32), y_dt)
     t0 = time.perf_counter()
     res = orc.loop_dispatch(og, M, E, K, cap)
-    orc.loop_combine(og, M, E, K, H, expert_y, ORACLE_DTYPE[spec.expert_y_dtype], ORACLE_DTYPE[spec.out_dtype], res.slot_map)
+    orc.loop_combine(og, M, E, K, H, expert_y, y_dt, out_dt, res.slot_map)
     return {"value": (time.perf_counter() - t0) * 1e6, "unit": "us", "cores": 1, "kind": "port",
             "sample": "one full step, python loops over tokens and picks (oracle.a2a_oracle.loop_*)"}  # fmt: skip
 
@@ -239,7 +313,7 @@ def counter_probe(spec, launches=3):
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a few eager dispatch and
     combine launches of the workload plus a plain elementwise copy of known size (1 GiB read,
     1 GiB written) whose counter reading calibrates the unit."""
-    from tests.all_to_all_utils import DeviceStep, expert_counts, generate, make_world
+    from pplx_kernels.workloads import DeviceStep, expert_counts, generate, make_world
 
     groups = generate(spec)
     cap = max(int(expert_counts(groups, spec.num_experts).max()), 1)
@@ -259,13 +333,29 @@ def counter_probe(spec, launches=3):
     world.destroy()
 
 
+def steps_for(name, steps_k):
+    """Timed steps per workload: the large prefills take milliseconds per step."""
+    if name == "C5":
+        return max(10, steps_k // 10)
+    if name == "C4":
+        return max(20, steps_k // 4)
+    return steps_k
+
+
+COMPACT_FIELDS = (
+    "workload", "tokens", "pairs", "buffer_sets", "steps_timed", "launch_form", "step_us", "bound_eager_step_us",
+    "graph_step_us", "dispatch_us", "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac",
+)  # fmt: skip
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2")
-    ap.add_argument("--all", action="store_true", help="also measure C1, C3, C4, C5 (reported under 'other_workloads')")
+    ap.add_argument("--workload", default="C2", help="the headline workload (value, roofline, cpu_baseline)")
+    ap.add_argument("--only", action="store_true", help="measure the headline workload alone (profiling runs)")
+    ap.add_argument("--all", action="store_true", help="accepted for compatibility: every workload is measured by default")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-probe", action="store_true", help="few eager launches + a calibration copy, for rocprofv3 --pmc")
     args = ap.parse_args()
@@ -281,7 +371,7 @@ def main() -> None:
         sys.exit(2)
     torch.cuda.set_device(0)
     from pplx_kernels import ops
-    from tests.all_to_all_utils import baseline_configs
+    from pplx_kernels.workloads import baseline_configs
 
     ops.load_library()  # fail loudly here if the HIP library is missing
     specs = baseline_configs()
@@ -289,71 +379,41 @@ def main() -> None:
     if args.counter_probe:
         counter_probe(spec)
         return
-    main_res, groups, steps = measure_workload(args.workload, spec, args.steps, args.warmup)
+    main_res, groups, steps = measure_workload(args.workload, spec, steps_for(args.workload, args.steps), args.warmup)
+    roofline = combine_kernel_roofline(args.workload, spec, steps, main_res["combine_bytes"], args.steps)
+    del steps
+    torch.cuda.empty_cache()
 
-    # Roofline of the dominant kernel: graphs holding back-to-back combine_gather launches
-    # only (the table bind is recorded once per graph), rotating buffer sets.
-    from tests.all_to_all_utils import make_world
+    workloads = {args.workload: {k: main_res[k] for k in COMPACT_FIELDS}}
+    if not args.only:
+        # the 8192-token prefill (the >= 60 % target) first, then the rest
+        for name in ("C5", "C4", "C3", "C1"):
+            if name == args.workload:
+                continue
+            res, _, st = measure_workload(name, specs[name], steps_for(name, args.steps), min(args.warmup, 5))
+            del st
+            torch.cuda.empty_cache()
+            workloads[name] = {k: res[k] for k in COMPACT_FIELDS}
+            if name == "C1" and not args.no_cpu:
+                workloads[name]["cpu_literal_loops"] = cpu_literal_loops(specs[name])
 
-    world = make_world(spec, group_name="bench-roofline")
-    stream = torch.cuda.Stream()
-    n_sets = len(steps)
-    launches_per_graph = 8
-
-    def many_combines(st):
-        def body():
-            for _ in range(launches_per_graph):
-                st.combine_world(world)
-        return body
-
-    with torch.cuda.stream(stream):
-        for st in steps:
-            st.dispatch_world(world)  # slot map of this world
-        stream.synchronize()
-    # combine reads the world's slot map, identical for every buffer set (same routing)
-    k_graphs = [capture(world, stream, many_combines(st)) for st in steps]
-    reps = max(1, args.steps // (n_sets * launches_per_graph))
-    per_graph_us = time_graphs(k_graphs, list(range(n_sets)), stream, 2, reps)
-    kernel_us = per_graph_us / launches_per_graph
-    for g in k_graphs:
-        g.destroy()
-    world.destroy()
-    comb_b = main_res["combine_bytes"]
-    roofline = {
-        "kernel": "combine_gather<bf16,bf16>",
-        "bound": "hbm",
-        "achieved": comb_b / kernel_us / 1e3,
-        "peak": HBM_PEAK_GBPS,
-        "unit": "GB/s",
-        "frac": comb_b / kernel_us / 1e3 / HBM_PEAK_GBPS,
-        "traffic": MEASURED_COMBINE_TRAFFIC_BYTES.get(args.workload),
-        "bytes_per_launch": comb_b,
-        "avg_launch_us": kernel_us,
-        "launches_timed": reps * n_sets * launches_per_graph,
-    }
-
-    # A step can be launched two ways: replaying a captured hipGraph, or two eager library calls
-    # on arguments packed once (LoopbackWorld.bind).  Both run the same kernels on the same
-    # rotating buffer sets; the headline is the faster one and says which (on this stack one
-    # hipGraphLaunch call costs more host time than two eager launches).
-    graph_us, bound_us = main_res["step_us"], main_res["bound_eager_step_us"]
-    best_us = min(graph_us, bound_us)
-    timed = (
-        f"{'eager launches of a bound step (LoopbackWorld.bind)' if bound_us <= graph_us else 'hipGraph replay'}"
-        f" of dispatch+combine, rotating buffer sets; hipGraph replay {graph_us:.1f} us, bound eager {bound_us:.1f} us"
-    )
+    form = {
+        "bound_eager": "eager launches of a bound step (LoopbackWorld.bind: pplx_a2a_world_dispatch + _combine on "
+        "arguments packed once)",
+        "graph_replay": f"one captured hipGraph replayed {GRAPH_REPLAYS_C3} times",
+    }[main_res["launch_form"]]
     result = {
         "metric": "dispatch+combine latency (us) and achieved HBM GB/s, DSv3 shape 128 tok/rank, 1 GPU",
-        "value": best_us,
+        "value": main_res["step_us"],
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": best_us / 1e3,
+        "ms_per_step": main_res["step_us"] / 1e3,
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "fp8_e4m3 rows + f32 block scales moved as bytes; combine bf16 in, f32 accumulate, bf16 out",
         "data": "synthetic",
         "config": {
             "workload": spec.name,
@@ -364,27 +424,15 @@ def main() -> None:
             "tokens_per_rank": spec.max_num_tokens,
             "in_dtype": str(spec.in_dtype).replace("torch.", ""),
             "out_dtype": str(spec.out_dtype).replace("torch.", ""),
-            "timed": timed,
+            "timed": f"{form}, rotating buffer sets; the same step as a hipGraph replay takes "
+            f"{main_res['graph_step_us']:.1f} us, as bound eager launches {main_res['bound_eager_step_us']:.1f} us",
         },
         "roofline": roofline,
+        "workloads": workloads,
         "detail": main_res,
     }
     if not args.no_cpu:
-        del steps
-        torch.cuda.empty_cache()
         result["cpu_baseline"] = cpu_baseline(spec, groups)
-    if args.all:
-        others = {}
-        for name, sp in specs.items():
-            if name == args.workload:
-                continue
-            k = args.steps if name != "C5" else max(8, args.steps // 10)
-            others[name], _, st = measure_workload(name, sp, k, min(args.warmup, 5))
-            del st
-            torch.cuda.empty_cache()
-            if name == "C1" and not args.no_cpu:
-                others[name]["cpu_literal_loops"] = cpu_literal_loops(sp)
-        result["other_workloads"] = others
     print(json.dumps(result))
 
 
