@@ -180,6 +180,23 @@ int check_config(const pplx_a2a_config_t &c) {
   return PPLX_A2A_OK;
 }
 
+// LDS bytes per CU of `device` (0 when the runtime will not say), looked up once per device.
+uint32_t lds_per_cu_of(int device) {
+  static std::mutex mu;
+  static int cached[64];
+  static bool known[64];
+  if (device < 0 || device >= 64) return 0;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!known[device]) {
+    int bytes = 0;
+    if (hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device) != hipSuccess)
+      bytes = 0;
+    cached[device] = bytes > 0 ? bytes : 0;
+    known[device] = true;
+  }
+  return (uint32_t)cached[device];
+}
+
 // The geometry part of a WorldDev (everything but the pointers) for a checked configuration.
 void fill_geometry(const pplx_a2a_config_t &cfg, WorldDev &d) {
   d.R = cfg.world_size;
@@ -677,6 +694,7 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
   w->device = device;
   WorldDev &d = w->dev;
   fill_geometry(*cfg, d);
+  d.lds_per_cu = lds_per_cu_of(device);
 
   auto cleanup = [&]() {
     for (hipEvent_t ev : w->rank_events) (void)hipEventDestroy(ev);
@@ -910,6 +928,7 @@ int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
     return fail(PPLX_A2A_INVALID_ARGUMENT, "device %d out of range (%d visible)", device, n_dev);
   DeviceScope scope(device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", device);
+  d.lds_per_cu = lds_per_cu_of(device);
   void *base = nullptr;
   LAUNCH_TRY(static_scratch_address(device, &base));
   uint8_t *scratch = static_cast<uint8_t *>(base);

@@ -72,12 +72,14 @@ __device__ __forceinline__ PPLX_GLOBAL V *as_global(V *p) {
 //                  tokens: 18.9 instead of 22.6 us; from about 240 MB per step on it is the
 //                  slowest of the three).
 // The compiler offers no builtin for the scoped forms, hence the asm; they are plain vector stores.
-enum class RowStore { kStream, kStreamThrough, kKeep };
+enum class RowStore { kStream, kStreamThrough, kKeep, kPlain };
 
 template <RowStore POLICY, typename V>
 __device__ __forceinline__ void row_store(V v, PPLX_GLOBAL V *p) {
   static_assert(sizeof(V) == 16 || sizeof(V) == 4, "row_store: 4- or 16-byte values");
-  if constexpr (POLICY == RowStore::kStream) {
+  if constexpr (POLICY == RowStore::kPlain) {
+    *p = v;
+  } else if constexpr (POLICY == RowStore::kStream) {
     __builtin_nontemporal_store(v, p);
   } else if constexpr (POLICY == RowStore::kStreamThrough) {
     if constexpr (sizeof(V) == 16) {

@@ -73,6 +73,7 @@ struct WorldDev {
   uint32_t S;        // fp32 scales per row
   uint32_t tile_chunks;  // 64-token chunks per routing tile of a whole-step dispatch
   uint32_t num_tiles;    // ceil(G * M / (64 * tile_chunks))
+  uint32_t lds_per_cu;   // bytes of LDS a CU has (0 = unknown): launches use it to cap residency
   DispatchRank *drank;   // [R]
   CombineRank *crank;    // [R]
   uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile; after route_scan the
@@ -127,7 +128,7 @@ constexpr uint32_t kInlineRanks = 64;
 constexpr uint32_t kBindBatch = 64;
 // Steps of at most this many virtual tokens (DP groups x max_num_tokens) dispatch in one fused
 // launch.
-constexpr uint32_t kFusedMaxTokens = 16384;
+constexpr uint32_t kFusedMaxTokens = 3072;
 // A fused launch whose rows (all picks of all tokens) stay within this many bytes stores them
 // write-through into the 256 MB last-level cache instead of streaming them past it.
 constexpr uint64_t kWriteThroughMaxBytes = 128ull << 20;

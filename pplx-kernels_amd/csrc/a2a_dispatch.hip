@@ -44,6 +44,8 @@ __global__ __launch_bounds__(256) void bind_rows(Row *table, Batch b) {
   }
 }
 
+// Launched as one-wave workgroups whose dynamic LDS size caps how many of them a CU holds at a
+// time (see launch_scatter_t); the kernel itself does not touch LDS.
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
   const uint32_t lane = lane_id();
@@ -67,7 +69,10 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   }
   const uint32_t k0 = part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  store_row<NV, EXACT, RowStore::kStreamThrough>(w, src, t, lane, dst, k0, k1, regs);
+  // Rows stream past the caches; the 4-byte-per-lane scale rows are written through into the
+  // last-level cache instead, where the partial lines of neighbouring rows meet before they go
+  // to HBM (3-4 % of the kernel's time at 224-byte scale rows).
+  store_row<NV, EXACT, RowStore::kStreamThrough, RowStore::kKeep>(w, src, t, lane, dst, k0, k1, regs);
 }
 
 // Threads of a dispatch_fused workgroup: 16 waves (fewer, larger workgroups repeat less
@@ -404,6 +409,24 @@ uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
   return ksplit;
 }
 
+// Scatter waves a CU should hold at a time (0 = as many as fit).
+// Measured on 8 x 4096 tokens (us at 32 = full occupancy / 3 / 4 / 6 / 8 / 12 waves per CU):
+//   59 KiB stored per wave (DSv3 fp8, top-8)   449 / 418 / 441 / 446 / 444 / 437
+//   32 KiB (bf16 2048, top-8)                  227 / 207 / 217 / 219 / 220 / 223
+//   16 KiB (bf16 4096, top-2)                  170 / 179 / 153 / 163 / 165 / 167
+//    8 KiB (bf16 512, top-8)                    65 / 126 /  79 /  64 /  60 /  61
+//    4 KiB (bf16 1024, top-2)                   46 / 110 /  71 /  59 /  53 /  49
+// A wave's loads and launch are dead time for the stores, so the less a wave stores the more
+// of them it takes to keep the CU's stores going.
+uint32_t scatter_waves_per_cu(const WorldDev &w, uint32_t picks_per_wave) {
+  if (w.lds_per_cu == 0) return 0;
+  const uint64_t stored = (uint64_t)picks_per_wave * (w.Hb + 4ull * w.S);
+  if (stored >= 24 * 1024) return 3;
+  if (stored >= 12 * 1024) return 4;
+  if (stored >= 6 * 1024) return 8;
+  return 0;
+}
+
 template <class DT>
 int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
@@ -414,8 +437,17 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint32_t ksplit = pick_ksplit(w, kWave);
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
   const uint64_t waves = (uint64_t)tokens * ksplit;
-  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
-  const uint32_t lds = 0;
+  // One wave per workgroup, and few of them per CU at a time.  A wave reads one row and then
+  // has up to K rows of stores to issue; HBM takes those stores best when a CU sends the rows of
+  // three or four waves at a time rather than those of thirty-two interleaved (measured: 8 x
+  // <= 8192 DSv3 fp8 tokens, top-8: 474 us at full occupancy, 457 / 447 / 459 us at 2 / 3 / 4
+  // waves per CU; 8 x 4096 bf16 tokens of 8 KiB, top-2: 164 us at full occupancy, 149 / 146 us
+  // at 3 / 4).  The hardware has no such knob, so each workgroup asks for a share of the CU's
+  // LDS that only that many fit into.
+  const uint32_t waves_per_cu = scatter_waves_per_cu(w, kper);
+  uint32_t lds = waves_per_cu ? (w.lds_per_cu / waves_per_cu) & ~1023u : 0u;
+  if (lds > 65536u) lds = 65536u;
+  const dim3 grid((uint32_t)waves), block(kWave);
 #define PPLX_ROW_KERNEL_ARGS ksplit, kper
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL)                                                    \
   do {                                                                                           \
@@ -476,9 +508,11 @@ uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
 
 bool dispatch_is_fused(const WorldDev &w) {
   // Every workgroup recounts all earlier tokens (work that grows with the square of the token
-  // count and sits on the ALU), so the one-launch form pays while that stays hidden behind the
-  // row traffic: measured against the three-launch form at 7 KiB rows it wins by 8 % (K = 8)
-  // and 4 % (K = 2) at 16384 tokens and loses from 32768 on.
+  // count) and all sixteen waves of a workgroup store at once, while the scatter of the
+  // three-to-four-launch form keeps few storing waves per CU.  Measured at 7 KiB rows, top-8, 8
+  // ranks (one launch / routing + scatter): 2048 tokens 24 / 42 us, 4096 tokens 61.5 / 58.8 us,
+  // 8192 tokens 109 / 100 us: the one-launch form pays while the routing launches (about 16 us of
+  // latency) weigh more than the scatter's better rate.
   const uint64_t tokens = (uint64_t)w.G * w.M;
   return tokens <= kFusedMaxTokens && row_has_register_variant(w) && fused_lds_bytes(w, 16, true) <= 60 * 1024;
 }

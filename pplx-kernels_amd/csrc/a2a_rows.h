@@ -68,7 +68,7 @@ __device__ __forceinline__ Destination resolve_destination(const WorldDev &w, co
 }
 
 // Second half: lane k holds the destination of pick k; the row is stored for picks [k0, k1).
-template <int NV, bool EXACT, RowStore POLICY = RowStore::kStream>
+template <int NV, bool EXACT, RowStore POLICY = RowStore::kStream, RowStore SCALE_POLICY = POLICY>
 __device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank &src, uint32_t t,
                                           uint32_t lane, Destination dst, uint32_t k0, uint32_t k1,
                                           RowRegs<NV> &regs) {
@@ -93,7 +93,7 @@ __device__ __forceinline__ void store_row(const WorldDev &w, const DispatchRank 
     if (S) {
       PPLX_GLOBAL float *sout = global_ptr<float>(read_lane64(dst.scale, k));
       const int64_t step = (int64_t)read_lane64((uint64_t)dst.scale_step, k);
-      if (lane < S) row_store<POLICY>(regs.sc, sout + (int64_t)lane * step);
+      if (lane < S) row_store<SCALE_POLICY>(regs.sc, sout + (int64_t)lane * step);
       if (S > kWave) {
         const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
         for (uint32_t j = lane + kWave; j < S; j += kWave) {

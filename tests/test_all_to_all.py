@@ -293,7 +293,7 @@ def test_baseline_config_full_size(cfg, api):
 
 
 def test_c4_reduced_against_oracle():
-    # more than 16384 virtual tokens: routing tiles + scatter, as at full size
+    # more than 3072 virtual tokens: routing tiles + scatter, as at full size
     spec = dataclasses.replace(baseline_configs()["C4"], max_num_tokens=2100, hidden_dim=256)
     groups = generate(spec)
     cap = int(expert_counts(groups, spec.num_experts).max())
@@ -413,7 +413,7 @@ def test_combine_dtype_matrix(y_dtype, out_dtype):
     "E,K,M,R",
     [
         (512, 8, 300, 8), (1024, 4, 130, 4), (8, 8, 70, 2), (4, 1, 5, 1), (64, 6, 1500, 2), (2048, 2, 40, 2),
-        # beyond 16384 virtual tokens the step takes the routing-tile kernels and the scatter
+        # beyond 3072 virtual tokens the step takes the routing-tile kernels and the scatter
         (512, 8, 2100, 8), (2048, 2, 8300, 2), (64, 6, 4200, 4), (4, 1, 17000, 1), (1024, 3, 4200, 4),
         # the limits of the build: 64 picks per token, 5440 experts (one 64-token chunk per routing tile)
         (128, 64, 20, 4), (5440, 64, 3, 2),
@@ -421,7 +421,7 @@ def test_combine_dtype_matrix(y_dtype, out_dtype):
 )  # fmt: skip
 def test_geometries(E, K, M, R):
     """Expert counts that change the routing tile shape, several tiles, K = E, K = 1, in both
-    forms of dispatch (one launch up to 16384 virtual tokens, three beyond)."""
+    forms of dispatch (one launch up to 3072 virtual tokens, three beyond)."""
     spec = _small_spec(name=f"geo{E}", world_size=R, num_experts=E, experts_per_token=K, max_num_tokens=M, hidden_dim=128)
     run_and_check(spec, generate(spec), use_numpy=True)
 
@@ -526,7 +526,7 @@ def test_row_sizes(hidden_bytes):
 
 @pytest.mark.parametrize("hidden_bytes", [16, 48, 1024 + 16, 4096, 7168, 10240, 12288, 14336, 16384, 16384 + 32])
 def test_row_sizes_in_the_scatter_kernel(hidden_bytes):
-    """The same row shapes where dispatch is routing tiles + scatter (> 16384 virtual tokens)."""
+    """The same row shapes where dispatch is routing tiles + scatter (> 3072 virtual tokens)."""
     spec = _small_spec(
         name=f"srow{hidden_bytes}", hidden_dim=hidden_bytes // 2, max_num_tokens=4200, experts_per_token=2,
         tokens="uniform",

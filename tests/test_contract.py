@@ -121,7 +121,7 @@ def _check_with_repeats_dropped(step, after_combine: bool):
         dict(name="dup-fp8", in_dtype=FP8, hidden_dim=512, experts_per_token=8, num_experts=32),
         dict(name="dup-odd-k", experts_per_token=3),
         dict(name="dup-top12", experts_per_token=12, num_experts=32),
-        # more than 16384 virtual tokens: routing tiles + scatter
+        # more than 3072 virtual tokens: routing tiles + scatter
         dict(name="dup-tiles", max_num_tokens=4200, experts_per_token=2),
     ],
     ids=lambda kw: kw["name"],

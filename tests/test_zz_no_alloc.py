@@ -122,7 +122,7 @@ def test_static_step_matches_the_world_path_on_calls_in_a_row():
     for g in groups:
         g.n = g.n // 3
     _compare(spec, groups, fault_word)
-    # 4. more than 16384 virtual tokens: the routing tiles' counts live in the array too
+    # 4. more than 3072 virtual tokens: the routing tiles' counts live in the array too
     tiled = _spec(name="c", world_size=4, num_experts=16, experts_per_token=2, hidden_dim=128,
                   max_num_tokens=4200, in_dtype=torch.bfloat16, dp_size=2)  # fmt: skip
     groups = generate(tiled)
