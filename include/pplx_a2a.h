@@ -159,10 +159,12 @@ uint32_t pplx_a2a_rank(const pplx_a2a_t *handle);
  * kernels; work a rank enqueues BETWEEN its own call and the last rank's call
  * is not ordered against the step.  The ranks of a captured step must share
  * one stream (PPLX_A2A_INVALID_STATE otherwise).
- * With SEND / RECV a call enqueues at once on its `stream`: every rank's SEND
- * must be enqueued before the first RECV, staging must have been reserved with
- * pplx_a2a_world_reserve_split (PPLX_A2A_INVALID_STATE otherwise), and ranks on
- * different streams order them themselves.
+ * SEND and RECV are collective in the same way, phase by phase: the last
+ * rank's SEND enqueues the sends of all ranks (inputs may be reused once it has
+ * returned, in stream order; no output is touched), the last rank's RECV the
+ * receives (outputs are those named by the RECV calls).  Every rank's SEND must
+ * come before the first RECV, and staging must have been reserved with
+ * pplx_a2a_world_reserve_split (PPLX_A2A_INVALID_STATE otherwise).
  * Without bound_m, m may not exceed max_num_tokens
  * (csrc/all_to_all/intranode_dispatch.cu:65); the members of a DP group must
  * pass the same m. */

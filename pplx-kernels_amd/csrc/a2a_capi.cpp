@@ -132,7 +132,7 @@ struct pplx_a2a_world {
   SplitDev split{};
   bool split_ready = false;
   uint32_t split_y_elem_bytes = 0;  // widest expert_y element the combine staging holds
-  std::vector<uint8_t> dsend, drecv, csend, crecv, group_routed;
+  std::vector<uint8_t> dsend, drecv, csend, crecv;
   uint32_t n_dsend = 0, n_drecv = 0, n_csend = 0, n_crecv = 0;
   int split_in_dtype = -1;
 };
@@ -213,8 +213,13 @@ void fill_geometry(const pplx_a2a_config_t &cfg, WorldDev &d) {
   // is one workgroup, and routing is a chain of short launches that only parallelism shortens),
   // at most 16 chunks of 64 tokens, and such that the LDS tables fit 64 KiB.
   const uint64_t step_chunks = ((uint64_t)d.G * d.M + kWave - 1) / kWave;
+  // A step of up to 1024 tokens is a single tile (one launch instead of three).
   d.tile_chunks = 1;
-  while (d.tile_chunks < 16 && step_chunks / d.tile_chunks > 256) d.tile_chunks *= 2;
+  if (step_chunks <= 16) {
+    while (d.tile_chunks < step_chunks) d.tile_chunks *= 2;
+  } else {
+    while (d.tile_chunks < 16 && step_chunks / d.tile_chunks > 256) d.tile_chunks *= 2;
+  }
   while (d.tile_chunks > 1 && route_lds_bytes(d.E, d.tile_chunks) > 65536u) d.tile_chunks /= 2;
   const uint64_t tile_tokens = (uint64_t)d.tile_chunks * kWave;
   d.num_tiles = (uint32_t)(((uint64_t)d.G * d.M + tile_tokens - 1) / tile_tokens);
@@ -477,13 +482,9 @@ uint64_t round_up(uint64_t x, uint64_t to) { return (x + to - 1) / to * to; }
 void free_split(pplx_a2a_world &w) {
   SplitDev &sp = w.split;
   (void)hipFree(sp.stage_x);
-  (void)hipFree(sp.gtile_cnt);
-  (void)hipFree(sp.gslot);
   (void)hipFree(sp.gexp);
   (void)hipFree(sp.gcnt);
   (void)hipFree(sp.goff);
-  (void)hipFree(sp.gbase);
-  (void)hipFree(sp.gntok);
   (void)hipFree(sp.stage_y);
   sp = SplitDev{};
   w.split_ready = false;
@@ -503,24 +504,14 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
     if (w.n_arrived_dispatch != 0 || w.n_arrived_combine != 0)
       return fail(PPLX_A2A_INVALID_STATE, "a step is being assembled");
     sp.token_stride = (uint32_t)round_up((uint64_t)d.Hb + 4ull * d.S + 4, 16);
-    // One group's SEND routes max_num_tokens tokens: a single tile when they fit one workgroup.
-    sp.tile_chunks = 1;
-    while (sp.tile_chunks < 16 && (uint64_t)sp.tile_chunks * kWave < d.M) sp.tile_chunks *= 2;
-    while (sp.tile_chunks > 1 && route_lds_bytes(d.E, sp.tile_chunks) > 65536u) sp.tile_chunks /= 2;
-    const uint64_t tile_tokens = (uint64_t)sp.tile_chunks * kWave;
-    sp.tiles_per_group = (uint32_t)((d.M + tile_tokens - 1) / tile_tokens);
     struct Alloc {
       void **ptr;
       size_t bytes;
     } allocs[] = {
         {reinterpret_cast<void **>(&sp.stage_x), pairs * sp.token_stride},
-        {reinterpret_cast<void **>(&sp.gtile_cnt), sizeof(uint32_t) * (size_t)d.G * sp.tiles_per_group * d.E},
-        {reinterpret_cast<void **>(&sp.gslot), sizeof(uint32_t) * pairs},
         {reinterpret_cast<void **>(&sp.gexp), sizeof(uint32_t) * pairs},
-        {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.G * d.E},
-        {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.G * d.E},
-        {reinterpret_cast<void **>(&sp.gbase), sizeof(uint32_t) * (size_t)d.G * d.E},
-        {reinterpret_cast<void **>(&sp.gntok), sizeof(uint32_t) * (size_t)d.G},
+        {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.E},
+        {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.E},
     };
     for (const Alloc &a : allocs) {
       hipError_t err = hipMalloc(a.ptr, a.bytes);
@@ -535,7 +526,6 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
     w.drecv.assign(d.R, 0);
     w.csend.assign(d.R, 0);
     w.crecv.assign(d.R, 0);
-    w.group_routed.assign(d.G, 0);
     w.split_ready = true;
   }
   if (y_elem_bytes > w.split_y_elem_bytes) {
@@ -564,59 +554,104 @@ int need_split(const pplx_a2a_world &w, uint32_t y_elem_bytes) {
   return PPLX_A2A_OK;
 }
 
-int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, int mode, void *stream) {
+// Split mode is collective phase by phase: the calls of a phase are recorded and the last
+// rank's call enqueues the phase for all ranks (on its stream, ordered against the streams the
+// other ranks called on).  SEND reads the inputs recorded by the SEND calls, RECV writes the
+// outputs named by the RECV calls.
+int run_split_dispatch(pplx_a2a_world &w, int mode, void *stream) {
   DeviceScope scope(w.device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
+  if (st) return st;
+  settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
+  const DispatchRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_dispatch.data() : nullptr;
+  if (!inline_rows) {
+    st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
+                                                      w.bound_dispatch_valid, false, launch_bind_dispatch, stream);
+    if (st) return st;
+  }
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    st = check_groups(w.dev, w.pend_dispatch.data());
+    if (st) return st;
+    ProfilerRange range("dispatch send");
+    LAUNCH_TRY(launch_split_dispatch_send(w.dev, w.split, inline_rows, pick_vector_of(w), stream));
+  } else {
+    ProfilerRange range("dispatch recv");
+    LAUNCH_TRY(launch_split_dispatch_recv(w.dev, w.split, inline_rows, stream));
+  }
+  return PPLX_A2A_OK;
+}
+
+int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, int mode, void *stream) {
   if (w.n_arrived_dispatch != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv dispatch step is still being assembled");
   int st = need_split(w, 0);
   if (st) return st;
   const uint32_t R = w.dev.R;
-  ProfilerRange range(mode == PPLX_A2A_SPLIT_SEND ? "dispatch send" : "dispatch recv");
   if (mode == PPLX_A2A_SPLIT_SEND) {
-    if (w.n_drecv != 0)
+    if (w.n_drecv != 0 || w.n_dsend == R)
       return fail(PPLX_A2A_INVALID_STATE,
                   "rank %u: dispatch SEND of the next step before every rank's RECV of this one", rank);
     if (w.dsend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called dispatch SEND twice", rank);
-    // The first member of a DP group to send routes the group (its members hold the same tokens).
-    const uint32_t g = rank / w.dev.dp;
-    if (!w.group_routed[g]) {
-      LAUNCH_TRY(launch_split_route(w.dev, w.split, row, rank, pick_vector_for(w.dev.K, row.indices), stream));
-      w.group_routed[g] = 1;
-    }
-    LAUNCH_TRY(launch_split_dispatch_send(w.dev, w.split, row, rank, stream));
+    w.pend_dispatch[rank] = row;
+    w.stream_dispatch[rank] = stream;
     w.dsend[rank] = 1;
-    ++w.n_dsend;
-    return PPLX_A2A_OK;
+    if (++w.n_dsend < R) return PPLX_A2A_OK;
+    st = run_ordered(w, w.stream_dispatch, stream, [&] { return run_split_dispatch(w, mode, stream); });
+    if (st) {  // nothing was sent: the step starts over
+      std::fill(w.dsend.begin(), w.dsend.end(), 0);
+      w.n_dsend = 0;
+    }
+    return st;
   }
   if (w.n_dsend != R)
     return fail(PPLX_A2A_INVALID_STATE,
                 "rank %u: dispatch RECV before every rank's SEND (%u of %u sent); in a loopback "
                 "world all SENDs must be enqueued first", rank, w.n_dsend, R);
   if (w.drecv[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called dispatch RECV twice", rank);
-  LAUNCH_TRY(launch_split_dispatch_recv(w.dev, w.split, row, rank, w.n_drecv == 0, stream));
+  w.pend_dispatch[rank] = row;
+  w.stream_dispatch[rank] = stream;
   w.drecv[rank] = 1;
-  if (++w.n_drecv == R) {
-    std::fill(w.dsend.begin(), w.dsend.end(), 0);
-    std::fill(w.drecv.begin(), w.drecv.end(), 0);
-    std::fill(w.group_routed.begin(), w.group_routed.end(), 0);
-    w.n_dsend = w.n_drecv = 0;
+  if (++w.n_drecv < R) return PPLX_A2A_OK;
+  std::fill(w.dsend.begin(), w.dsend.end(), 0);
+  std::fill(w.drecv.begin(), w.drecv.end(), 0);
+  w.n_dsend = w.n_drecv = 0;
+  return run_ordered(w, w.stream_dispatch, stream, [&] { return run_split_dispatch(w, mode, stream); });
+}
+
+int run_split_combine(pplx_a2a_world &w, int mode, int in_dtype, int out_dtype, void *stream) {
+  DeviceScope scope(w.device);
+  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
+  unsigned long long session = 0;
+  int st = capture_session(stream, &session);
+  if (st) return st;
+  settle_mirror(w, session, w.bind_capture_combine, w.bound_combine_valid);
+  const CombineRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_combine.data() : nullptr;
+  if (!inline_rows) {
+    st = flush_table<CombineRank, BindCombineBatch>(w, w.pend_combine, w.bound_combine, w.bound_combine_valid,
+                                                    false, launch_bind_combine, stream);
+    if (st) return st;
+  }
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    ProfilerRange range("combine send");
+    LAUNCH_TRY(launch_split_combine_send(w.dev, w.split, inline_rows, in_dtype, stream));
+  } else {
+    ProfilerRange range("combine recv");
+    LAUNCH_TRY(launch_split_combine_recv(w.dev, w.split, inline_rows, in_dtype, out_dtype, stream));
   }
   return PPLX_A2A_OK;
 }
 
 int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int in_dtype, int out_dtype,
                   int mode, void *stream) {
-  DeviceScope scope(w.device);
-  if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   if (w.n_arrived_combine != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv combine step is still being assembled");
   int st = need_split(w, (uint32_t)dtype_size(in_dtype));
   if (st) return st;
   const uint32_t R = w.dev.R;
-  ProfilerRange range(mode == PPLX_A2A_SPLIT_SEND ? "combine send" : "combine recv");
   if (mode == PPLX_A2A_SPLIT_SEND) {
-    if (w.n_crecv != 0)
+    if (w.n_crecv != 0 || w.n_csend == R)
       return fail(PPLX_A2A_INVALID_STATE,
                   "rank %u: combine SEND of the next step before every rank's RECV of this one", rank);
     if (w.csend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine SEND twice", rank);
@@ -624,10 +659,17 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
       return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
     w.split_in_dtype = in_dtype;
     w.split.y_row_bytes = (uint64_t)w.dev.H * dtype_size(in_dtype);
-    LAUNCH_TRY(launch_split_combine_send(w.dev, w.split, row, rank, in_dtype, stream));
+    w.pend_combine[rank] = row;
+    w.stream_combine[rank] = stream;
     w.csend[rank] = 1;
-    ++w.n_csend;
-    return PPLX_A2A_OK;
+    if (++w.n_csend < R) return PPLX_A2A_OK;
+    st = run_ordered(w, w.stream_combine, stream,
+                     [&] { return run_split_combine(w, mode, in_dtype, out_dtype, stream); });
+    if (st) {
+      std::fill(w.csend.begin(), w.csend.end(), 0);
+      w.n_csend = 0;
+    }
+    return st;
   }
   if (w.n_csend != R)
     return fail(PPLX_A2A_INVALID_STATE,
@@ -636,14 +678,18 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
   if (w.crecv[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine RECV twice", rank);
   if (w.split_in_dtype != in_dtype)
     return fail(PPLX_A2A_UNSUPPORTED, "combine RECV must use the expert_y dtype of the SEND phase");
-  LAUNCH_TRY(launch_split_combine_recv(w.dev, w.split, row, rank, in_dtype, out_dtype, stream));
+  if (w.n_crecv != 0 && w.combine_out_dtype != out_dtype)
+    return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
+  w.combine_out_dtype = out_dtype;
+  w.pend_combine[rank] = row;
+  w.stream_combine[rank] = stream;
   w.crecv[rank] = 1;
-  if (++w.n_crecv == R) {
-    std::fill(w.csend.begin(), w.csend.end(), 0);
-    std::fill(w.crecv.begin(), w.crecv.end(), 0);
-    w.n_csend = w.n_crecv = 0;
-  }
-  return PPLX_A2A_OK;
+  if (++w.n_crecv < R) return PPLX_A2A_OK;
+  std::fill(w.csend.begin(), w.csend.end(), 0);
+  std::fill(w.crecv.begin(), w.crecv.end(), 0);
+  w.n_csend = w.n_crecv = 0;
+  return run_ordered(w, w.stream_combine, stream,
+                     [&] { return run_split_combine(w, mode, in_dtype, out_dtype, stream); });
 }
 
 void reset_dispatch_arrivals(pplx_a2a_world &w) {

@@ -217,9 +217,12 @@ int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dty
 
 }  // namespace
 
-int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
-                              uint32_t rank, int in_dtype, int out_dtype, void *stream) {
-  return launch_combine_t(w, SingleCombine{row}, in_dtype, out_dtype, (hipStream_t)stream, rank, 1,
+int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
+                              int in_dtype, int out_dtype, void *stream) {
+  if (inline_rows)
+    return launch_combine_t(w, make_inline<true>(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream, 0,
+                            w.R, sp.stage_y, sp.y_row_bytes);
+  return launch_combine_t(w, HbmCombineT<true>{w.crank}, in_dtype, out_dtype, (hipStream_t)stream, 0, w.R,
                           sp.stage_y, sp.y_row_bytes);
 }
 

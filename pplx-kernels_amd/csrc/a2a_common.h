@@ -26,16 +26,20 @@ struct HbmDispatch {
   const DispatchRank *rows;
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
-struct InlineCombine {
-  static constexpr bool kStaged = false;
+// STAGED: combine reads the rows that combine SEND of split mode left in the world's staging
+// area instead of expert_y.
+template <bool STAGED> struct InlineCombineT {
+  static constexpr bool kStaged = STAGED;
   CombineRank rows[kInlineRanks];
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
-struct HbmCombine {
-  static constexpr bool kStaged = false;
+template <bool STAGED> struct HbmCombineT {
+  static constexpr bool kStaged = STAGED;
   const CombineRank *rows;
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
+typedef InlineCombineT<false> InlineCombine;
+typedef HbmCombineT<false> HbmCombine;
 
 // Pointers rebuilt from integers would be "flat" to the compiler; these casts say
 // that they are global memory, so that plain global_load / global_store are emitted.
@@ -134,19 +138,6 @@ template <> struct SettleAll<16> {
                    "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]),
                    "+v"(r[13]), "+v"(r[14]), "+v"(r[15]));
   }
-};
-
-// Split mode: a launch sees only the calling rank's arguments (its peers may not
-// have called yet), whatever rank index is asked for.
-struct SingleDispatch {
-  static constexpr bool kInline = false;
-  DispatchRank row;
-  __device__ __forceinline__ const DispatchRank &at(uint32_t) const { return row; }
-};
-struct SingleCombine {
-  static constexpr bool kStaged = true;  // rows come from the world's stage_y, not expert_y
-  CombineRank row;
-  __device__ __forceinline__ const CombineRank &at(uint32_t) const { return row; }
 };
 
 __device__ __forceinline__ uint32_t lane_id() {
@@ -248,8 +239,9 @@ inline InlineDispatch make_inline(const WorldDev &w, const DispatchRank *rows) {
   return t;
 }
 
-inline InlineCombine make_inline(const WorldDev &w, const CombineRank *rows) {
-  InlineCombine t{};
+template <bool STAGED = false>
+inline InlineCombineT<STAGED> make_inline(const WorldDev &w, const CombineRank *rows) {
+  InlineCombineT<STAGED> t{};
   for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
   return t;
 }

@@ -90,31 +90,25 @@ struct RouteSpan {
   uint32_t pick_vector;   // expert ids one load may fetch (4, 2 or 1)
   uint32_t *tile_cnt;     // [tiles][E]
   uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
-  // split mode only (one DP group per launch):
+  // split mode only:
   uint32_t *expert_out;   // [G * M][K] expert of every pair
-  uint32_t *counts_out;   // [E] rows per expert sent by the group
+  uint32_t *counts_out;   // [E] rows per expert
   uint32_t *offsets_out;  // [E] exclusive prefix of counts_out over experts
-  uint32_t *ntok_out;     // [1] tokens the group sent
 };
 
 // Device state of split send / recv mode: a two-hop path through staging that the world
-// owns.  dispatch SEND packs a group's rows, sorted by expert, into stage_x in the
-// reference's wire format  row | fp32 scales | u32 source token, padded to 16 bytes
-// (csrc/all_to_all/intranode.cpp:41-47, csrc/all_to_all/intranode_dispatch.cu:60-61,148-150);
-// dispatch RECV unpacks into the caller's expert-major outputs.  combine SEND copies expert
+// owns.  dispatch SEND packs every routed row, grouped by expert and ordered by slot, into
+// stage_x in the reference's wire format  row | fp32 scales | u32 source token, padded to 16
+// bytes (csrc/all_to_all/intranode.cpp:41-47, csrc/all_to_all/intranode_dispatch.cu:60-61,148-150);
+// dispatch RECV unpacks into the callers' expert-major outputs.  combine SEND copies expert
 // rows into stage_y, one row per (token, pick); combine RECV reduces them.
 struct SplitDev {
-  uint8_t *stage_x;        // [G][M * K rows][token_stride]
+  uint8_t *stage_x;        // [G * M * K rows][token_stride], expert e's rows start at goff[e]
   uint32_t token_stride;   // round_up(Hb + 4 S + 4, 16)
-  uint32_t tile_chunks;    // 64-token chunks per routing tile of one group's SEND
-  uint32_t tiles_per_group;
-  uint32_t *gtile_cnt;     // [G][tiles_per_group][E]
-  uint32_t *gslot;         // [G * M][K] row of a pair inside its (group, expert) run
-  uint32_t *gexp;          // [G * M][K] expert of a pair
-  uint32_t *gcnt;          // [G][E] rows group g sent to expert e
-  uint32_t *goff;          // [G][E] start of that run inside the group's staging area
-  uint32_t *gbase;         // [G][E] rows of expert e that come from groups before g
-  uint32_t *gntok;         // [G] tokens group g sent
+  uint32_t pad_;
+  uint32_t *gexp;          // [G * M][K] expert of a pair (num_experts = the pair has no row)
+  uint32_t *gcnt;          // [E] rows sent to expert e
+  uint32_t *goff;          // [E] exclusive prefix of gcnt over the experts
   uint8_t *stage_y;        // [G * M * K][y_row_bytes]
   uint64_t y_row_bytes;
 };
@@ -162,19 +156,15 @@ int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t
                     void *stream);
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
-// Split mode phases of one rank (`row` holds that rank's arguments of the call).
-// Routes the DP group of `rank` from that rank's indices (the members of a group hold the same
-// tokens, so the first member to send does it for the group); then every member packs its share.
-int launch_split_route(const WorldDev &w, const SplitDev &sp, const DispatchRank &row, uint32_t rank,
-                       uint32_t pick_vector, void *stream);
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
-                               uint32_t rank, void *stream);
-int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
-                               uint32_t rank, bool first_of_step, void *stream);
-int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
-                              uint32_t rank, int in_dtype, void *stream);
-int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
-                              uint32_t rank, int in_dtype, int out_dtype, void *stream);
+// Split mode phases, each for all ranks at once (`inline_rows` as above).
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                               uint32_t pick_vector, void *stream);
+int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                               void *stream);
+int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
+                              int in_dtype, void *stream);
+int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
+                              int in_dtype, int out_dtype, void *stream);
 // True when dispatch runs as the single fused launch for this geometry.
 bool dispatch_is_fused(const WorldDev &w);
 // LDS bytes the routing kernels need for a given geometry.

@@ -20,10 +20,10 @@ namespace {
 // An expert id repeated inside one token sets its bit once: the repeat takes no row, is not
 // counted, and is reported (kFaultDuplicateExpert).
 //
-// SPLIT = false: one launch routes every DP group and writes out_expert_num_tokens of the
-// owning ranks.  SPLIT = true: the launch routes the span of one DP group from the calling
-// rank's indices alone and leaves group-local results (slot inside (group, expert), expert of
-// each pair, rows per expert and their exclusive prefix over experts) for the later phases.
+// SPLIT = false: the launch writes out_expert_num_tokens of the owning ranks.  SPLIT = true
+// (dispatch SEND of split mode, which may not touch the outputs yet): the rows per expert go to
+// counts_out instead, together with their exclusive prefix over the experts and the expert of
+// every pair, for the pack / unpack phases.
 // ---------------------------------------------------------------------------
 
 // The token of this thread: which group and sender, whether its row of picks exists, and the
@@ -212,7 +212,6 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
       span.offsets_out[e] = running;
       running += span.counts_out[e];
     }
-    if (threadIdx.x == 0) *span.ntok_out = dispatch_group_tokens(w, tab, span.v_begin / w.M);
   }
 }
 

@@ -1,28 +1,39 @@
 // gfx950 kernels of split send / recv mode: two hops through world-owned staging in the
 // reference's wire format (row | scales | source token, 16-byte padded).
+//
+// The reference lets a rank send, compute, then receive (csrc/all_to_all/all_to_all.h:9-13,
+// csrc/all_to_all/bench_all_to_all.cpp:183-203).  In the loopback every phase is collective:
+// the ranks' calls of a phase are recorded, and the call of the last rank enqueues ONE launch
+// sequence for all of them, as in send+recv mode.
+//   dispatch SEND   routes the whole step (slot map, rows per expert and their prefix over the
+//                   experts) and packs every routed row into the staging area, grouped by
+//                   expert and ordered by slot: the expert-major receive buffer
+//   dispatch RECV   unpacks each expert's run of staged rows into the owning rank's outputs
+//   combine SEND    copies the expert_y row of every (token, pick) into the pair's staging row
+//                   (the reference copies it into the source rank's inbox,
+//                   csrc/all_to_all/intranode_combine.cu:77-111)
+//   combine RECV    is combine_gather reading the staged rows (a2a_combine.hip)
 #include "a2a_route.h"
 #include "a2a_rows.h"
 
 namespace pplx_amd {
 namespace {
 
-// ---------------------------------------------------------------------------
-// Split send / recv mode (two hops through world-owned staging).
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ uint8_t *stage_row(const WorldDev &w, const SplitDev &sp, uint32_t g,
-                                              uint32_t position) {
-  return sp.stage_x + ((uint64_t)g * w.M * w.K + position) * sp.token_stride;
+__device__ __forceinline__ uint8_t *stage_row(const SplitDev &sp, uint64_t position) {
+  return sp.stage_x + position * sp.token_stride;
 }
 
-// dispatch SEND, second half: one wave per token of the calling rank's share packs
-// row | scales | source token into the group's staging area, grouped by expert.
+// dispatch SEND, second half: one wave per token packs row | scales | source token for each of
+// its picks.  Lane k resolves pick k.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g, uint32_t member,
-                                                  SplitDev sp) {
+__global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev sp) {
   const uint32_t lane = lane_id();
-  const uint32_t t = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
-  if (t >= w.M || t % w.dp != member || t >= sp.gntok[g]) return;
-  const DispatchRank &src = tab.at(0);
+  const uint32_t v = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (g >= w.G) return;
+  if (t >= dispatch_group_tokens(w, tab, g)) return;
+  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
   const uint32_t nvec = w.Hb / 16;
   const PPLX_GLOBAL u32x4 *row =
       as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
@@ -40,11 +51,11 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g
   if (S) sc = srow[(int64_t)(lane < S ? lane : S - 1) * src.dp_xs_stride_elem];
   uint64_t dst = 0;
   if (lane < w.K) {
-    const size_t pair = ((size_t)g * w.M + t) * w.K + lane;
+    const size_t pair = (size_t)v * w.K + lane;
     const uint32_t e = as_global(sp.gexp)[pair];
-    if (e < w.E) {
-      dst = reinterpret_cast<uint64_t>(
-          stage_row(w, sp, g, as_global(sp.goff)[(size_t)g * w.E + e] + as_global(sp.gslot)[pair]));
+    const uint32_t slot = as_global(w.slot_map)[pair];
+    if (e < w.E && slot != kInvalidSlot) {
+      dst = reinterpret_cast<uint64_t>(stage_row(sp, (uint64_t)as_global(sp.goff)[e] + slot));
     }
   }
 #pragma unroll
@@ -69,56 +80,56 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, uint32_t g
   }
 }
 
-// First dispatch RECV of a step: rows of every expert that come from earlier groups.
-__global__ __launch_bounds__(256) void split_bases(WorldDev w, SplitDev sp) {
-  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= w.E) return;
-  uint32_t running = 0;
-  for (uint32_t g = 0; g < w.G; ++g) {
-    sp.gbase[(size_t)g * w.E + e] = running;
-    running += sp.gcnt[(size_t)g * w.E + e];
+// Rows beyond the register variants: plain streaming loops, one workgroup per token.
+template <class DT>
+__global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, SplitDev sp) {
+  const uint32_t v = blockIdx.x;
+  const uint32_t g = v / w.M;
+  const uint32_t t = v - g * w.M;
+  if (g >= w.G) return;
+  if (t >= dispatch_group_tokens(w, tab, g)) return;
+  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  const uint32_t nvec = w.Hb / 16;
+  const PPLX_GLOBAL u32x4 *row =
+      as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
+  const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
+  for (uint32_t k = 0; k < w.K; ++k) {
+    const size_t pair = (size_t)v * w.K + k;
+    const uint32_t e = as_global(sp.gexp)[pair];
+    const uint32_t slot = as_global(w.slot_map)[pair];
+    if (e >= w.E || slot == kInvalidSlot) continue;
+    uint8_t *p = stage_row(sp, (uint64_t)as_global(sp.goff)[e] + slot);
+    PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(p));
+    for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
+    PPLX_GLOBAL float *sout = as_global(reinterpret_cast<float *>(p + w.Hb));
+    for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) sout[j] = srow[(int64_t)j * src.dp_xs_stride_elem];
+    if (threadIdx.x == 0) *as_global(reinterpret_cast<uint32_t *>(p + w.Hb + 4ull * w.S)) = t;
   }
 }
 
-// ... and the slot map that combine reads: slot = rows from earlier groups + slot in the group.
-__global__ __launch_bounds__(256) void split_finalize(WorldDev w, SplitDev sp) {
-  const uint64_t pair = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (pair >= (uint64_t)w.G * w.M * w.K) return;
-  const uint32_t v = (uint32_t)(pair / w.K);
-  const uint32_t g = v / w.M;
-  const uint32_t t = v - g * w.M;
-  if (t >= sp.gntok[g]) return;
-  const uint32_t e = sp.gexp[pair];
-  w.slot_map[pair] = e < w.E ? sp.gbase[(size_t)g * w.E + e] + sp.gslot[pair] : kInvalidSlot;
-}
-
-// dispatch RECV of rank d: workgroup (local expert, group) copies that run of staged rows
-// into out_expert_x / out_expert_x_scale; blockIdx.y spreads long runs.
+// dispatch RECV: workgroup column blockIdx.x takes expert e; its run of staged rows goes to
+// out_expert_x / out_expert_x_scale of the owning rank, slot by slot; blockIdx.y spreads long
+// runs over workgroups.  The expert's count goes to out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t d, SplitDev sp,
-                                                    uint32_t write_through) {
+__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, SplitDev sp, uint32_t write_through) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const uint32_t el = blockIdx.x / w.G;
-  const uint32_t g = blockIdx.x - el * w.G;
-  const uint32_t e = d * w.L + el;
-  const DispatchRank &dst = tab.at(0);
-  const size_t ge = (size_t)g * w.E + e;
-  const uint32_t count = as_global(sp.gcnt)[ge], offset = as_global(sp.goff)[ge], base = as_global(sp.gbase)[ge];
-  if (g == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
-    const size_t last = (size_t)(w.G - 1) * w.E + e;
-    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] =
-        (int32_t)(as_global(sp.gbase)[last] + as_global(sp.gcnt)[last]);
+  const uint32_t e = blockIdx.x;
+  const uint32_t el = e % w.L;
+  const DispatchRank &dst = tab.at(e / w.L);
+  const uint32_t count = as_global(sp.gcnt)[e], offset = as_global(sp.goff)[e];
+  if (blockIdx.y == 0 && threadIdx.x == 0) {
+    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)count;
   }
   const uint32_t nvec = w.Hb / 16;
   const uint32_t S = w.S;
-  for (uint32_t i = blockIdx.y * (blockDim.x / kWave) + wave; i < count; i += gridDim.y * (blockDim.x / kWave)) {
-    const uint32_t slot = base + i;
+  const uint32_t waves = blockDim.x / kWave;
+  for (uint32_t slot = blockIdx.y * waves + wave; slot < count; slot += gridDim.y * waves) {
     if (slot >= dst.x_rows) {
       if (lane == 0) atomicOr(w.faults, kFaultRowDropped);
       continue;
     }
-    const uint8_t *src = stage_row(w, sp, g, offset + i);
+    const uint8_t *src = stage_row(sp, (uint64_t)offset + slot);
     const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
     PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
         dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
@@ -144,136 +155,110 @@ __global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, uint32_t
         const uint32_t j = lane + v * kWave;
         if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[v], out + j);
       }
-      if (lane < S) row_store<RowStore::kKeep>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
     } else {
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
         const uint32_t j = lane + v * kWave;
-        if (EXACT || j < nvec) row_store<RowStore::kStream>(x[v], out + j);
+        if (EXACT || j < nvec) row_store<RowStore::kStreamThrough>(x[v], out + j);
       }
-      if (lane < S) row_store<RowStore::kStream>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
     }
+    if (lane < S) row_store<RowStore::kKeep>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
     for (uint32_t j = lane + kWave; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
   }
 }
 
-// Rows beyond the register variants: plain streaming loops, one workgroup per staged row.
 template <class DT>
-__global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, uint32_t g, uint32_t member,
-                                                       SplitDev sp) {
-  const uint32_t t = blockIdx.x;
-  if (t >= w.M || t % w.dp != member || t >= sp.gntok[g]) return;
-  const DispatchRank &src = tab.at(0);
-  const uint32_t nvec = w.Hb / 16;
-  const u32x4 *row = reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row);
-  for (uint32_t k = 0; k < w.K; ++k) {
-    const size_t pair = ((size_t)g * w.M + t) * w.K + k;
-    const uint32_t e = sp.gexp[pair];
-    if (e >= w.E) continue;
-    uint8_t *p = stage_row(w, sp, g, sp.goff[(size_t)g * w.E + e] + sp.gslot[pair]);
-    u32x4 *out = reinterpret_cast<u32x4 *>(p);
-    for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
-    float *sout = reinterpret_cast<float *>(p + w.Hb);
-    for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) {
-      sout[j] = src.dp_xs[(int64_t)t * src.dp_xs_stride_row + (int64_t)j * src.dp_xs_stride_elem];
-    }
-    if (threadIdx.x == 0) *reinterpret_cast<uint32_t *>(p + w.Hb + 4ull * w.S) = t;
-  }
-}
-
-template <class DT>
-__global__ __launch_bounds__(256) void split_unpack_long(WorldDev w, DT tab, uint32_t d, SplitDev sp) {
-  const uint32_t el = blockIdx.x / w.G;
-  const uint32_t g = blockIdx.x - el * w.G;
-  const uint32_t e = d * w.L + el;
-  const DispatchRank &dst = tab.at(0);
-  const size_t ge = (size_t)g * w.E + e;
-  const uint32_t count = sp.gcnt[ge], offset = sp.goff[ge], base = sp.gbase[ge];
-  if (g == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
-    const size_t last = (size_t)(w.G - 1) * w.E + e;
-    dst.out_num_tokens[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)(sp.gbase[last] + sp.gcnt[last]);
+__global__ __launch_bounds__(256) void split_unpack_long(WorldDev w, DT tab, SplitDev sp) {
+  const uint32_t e = blockIdx.x;
+  const uint32_t el = e % w.L;
+  const DispatchRank &dst = tab.at(e / w.L);
+  const uint32_t count = as_global(sp.gcnt)[e], offset = as_global(sp.goff)[e];
+  if (blockIdx.y == 0 && threadIdx.x == 0) {
+    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)count;
   }
   const uint32_t nvec = w.Hb / 16;
-  for (uint32_t i = blockIdx.y; i < count; i += gridDim.y) {
-    const uint32_t slot = base + i;
+  for (uint32_t slot = blockIdx.y; slot < count; slot += gridDim.y) {
     if (slot >= dst.x_rows) {
       if (threadIdx.x == 0) atomicOr(w.faults, kFaultRowDropped);
       continue;
     }
-    const uint8_t *src = stage_row(w, sp, g, offset + i);
-    const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
-    u32x4 *out = reinterpret_cast<u32x4 *>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
-                                           (int64_t)slot * dst.x_stride_row);
+    const uint8_t *src = stage_row(sp, (uint64_t)offset + slot);
+    const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
+    PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
+        dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
     for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
-    const float *sin = reinterpret_cast<const float *>(src + w.Hb);
-    float *sout = dst.expert_xs + (int64_t)el * dst.xs_stride_expert + (int64_t)slot * dst.xs_stride_row;
+    const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
+    PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
+                              (int64_t)slot * dst.xs_stride_row;
     for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
   }
 }
 
-// combine SEND of rank d: one wave per (token, pick) whose expert d owns copies that
-// expert_y row into the pair's staging row (the reference copies it into the source
-// rank's inbox, csrc/all_to_all/intranode_combine.cu:77-111).
+// combine SEND: one wave per (token, pick) copies the expert_y row of the pick's expert into
+// the pair's staging row, eight 16-byte vectors per lane in flight.
 template <class CT>
-__global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, uint32_t d, SplitDev sp,
-                                                          uint32_t elem_bytes) {
+__global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, SplitDev sp, uint32_t elem_bytes) {
   const uint32_t lane = lane_id();
   const uint64_t pair = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
   if (pair >= (uint64_t)w.G * w.M * w.K) return;
   const uint32_t v = (uint32_t)(pair / w.K);
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  if (t >= sp.gntok[g]) return;
-  const uint32_t e = sp.gexp[pair];
-  if (e >= w.E || e / w.L != d) return;
-  const uint32_t slot = w.slot_map[pair];
-  const CombineRank &own = tab.at(0);
+  if (t >= combine_rank_tokens(w, tab.at(g * w.dp))) return;
+  const uint32_t e = as_global(sp.gexp)[pair];
+  const uint32_t slot = as_global(w.slot_map)[pair];
+  if (e >= w.E || slot == kInvalidSlot) return;
+  const CombineRank &own = tab.at(e / w.L);
   if (slot >= own.y_rows) {
     if (lane == 0) atomicOr(w.faults, kFaultBadSlot);
     return;
   }
   const uint8_t *src = reinterpret_cast<const uint8_t *>(own.expert_y) +
                        ((int64_t)(e % w.L) * own.y_stride_expert + (int64_t)slot * own.y_stride_row) * elem_bytes;
-  const u32x4 *row = reinterpret_cast<const u32x4 *>(src);
-  u32x4 *out = reinterpret_cast<u32x4 *>(sp.stage_y + pair * sp.y_row_bytes);
+  const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
+  PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(sp.stage_y + pair * sp.y_row_bytes));
   const uint32_t nvec = (uint32_t)(sp.y_row_bytes / 16);
-  for (uint32_t j = lane; j < nvec; j += kWave) out[j] = __builtin_nontemporal_load(row + j);
+  constexpr uint32_t kBatch = 8;
+  for (uint32_t j0 = 0; j0 < nvec; j0 += kBatch * kWave) {
+    u32x4 x[kBatch];
+#pragma unroll
+    for (uint32_t b = 0; b < kBatch; ++b) {
+      uint32_t j = j0 + b * kWave + lane;
+      j = j < nvec ? j : nvec - 1;
+      x[b] = __builtin_nontemporal_load(row + j);
+    }
+    SettleAll<kBatch>::of(x);
+#pragma unroll
+    for (uint32_t b = 0; b < kBatch; ++b) {
+      const uint32_t j = j0 + b * kWave + lane;
+      if (j < nvec) row_store<RowStore::kKeep>(x[b], out + j);
+    }
+  }
 }
 
-}  // namespace
-
-int launch_split_route(const WorldDev &w, const SplitDev &sp, const DispatchRank &row, uint32_t rank,
-                       uint32_t pick_vector, void *stream) {
-  typedef SingleDispatch DT;
-  const DT tab{row};
-  const uint32_t g = rank / w.dp;
+template <class DT>
+int launch_split_dispatch_send_t(const WorldDev &w, const SplitDev &sp, const DT &tab, uint32_t pick_vector,
+                                 hipStream_t s) {
   RouteSpan span{};
-  span.v_begin = g * w.M;
-  span.v_count = w.M;
-  span.tile_chunks = sp.tile_chunks;
+  span.v_begin = 0;
+  span.v_count = w.G * w.M;
+  span.tile_chunks = w.tile_chunks;
   span.pick_vector = pick_vector;
-  span.tile_cnt = sp.gtile_cnt + (size_t)g * sp.tiles_per_group * w.E;
-  span.slot_out = sp.gslot;
+  span.tile_cnt = w.tile_cnt;
+  span.slot_out = w.slot_map;
   span.expert_out = sp.gexp;
-  span.counts_out = sp.gcnt + (size_t)g * w.E;
-  span.offsets_out = sp.goff + (size_t)g * w.E;
-  span.ntok_out = sp.gntok + g;
-  return launch_route_t<DT, true>(w, tab, span, (hipStream_t)stream);
-}
-
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
-                               uint32_t rank, void *stream) {
-  typedef SingleDispatch DT;
-  hipStream_t s = (hipStream_t)stream;
-  const DT tab{row};
-  const uint32_t g = rank / w.dp, member = rank % w.dp;
+  span.counts_out = sp.gcnt;
+  span.offsets_out = sp.goff;
+  int err = launch_route_t<DT, true>(w, tab, span, s);
+  if (err) return err;
   const uint32_t lds = 0;
+  const uint32_t tokens = w.G * w.M;
   if (!row_has_register_variant(w)) {
-    hipLaunchKernelGGL(split_pack_long<DT>, dim3(w.M), dim3(256), 0, s, w, tab, g, member, sp);
+    hipLaunchKernelGGL(split_pack_long<DT>, dim3(tokens), dim3(256), 0, s, w, tab, sp);
     return (int)hipGetLastError();
   }
-  const dim3 grid((w.M + 3) / 4), block(256);
-#define PPLX_ROW_KERNEL_ARGS g, member, sp
+  const dim3 grid((tokens + 3) / 4), block(256);
+#define PPLX_ROW_KERNEL_ARGS sp
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(split_pack);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -281,35 +266,24 @@ int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const Disp
   return (int)hipGetLastError();
 }
 
-int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank &row,
-                               uint32_t rank, bool first_of_step, void *stream) {
-  typedef SingleDispatch DT;
-  hipStream_t s = (hipStream_t)stream;
-  const DT tab{row};
-  if (first_of_step) {
-    hipLaunchKernelGGL(split_bases, dim3((w.E + 255) / 256), dim3(256), 0, s, w, sp);
-    const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
-    hipLaunchKernelGGL(split_finalize, dim3((uint32_t)((pairs + 255) / 256)), dim3(256), 0, s, w, sp);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) return (int)err;
-  }
+template <class DT>
+int launch_split_dispatch_recv_t(const WorldDev &w, const SplitDev &sp, const DT &tab, hipStream_t s) {
   const uint32_t lds = 0;
-  // Row groups per (local expert, group) run: enough workgroups to cover the CUs even with few
-  // experts per rank, and a hot expert's long run is shared; never more than the run can use.
-  const uint32_t runs = w.L * w.G;
-  uint32_t spread = (2048 + runs - 1) / runs;
-  const uint32_t most = (w.M + 3) / 4;
-  if (spread > most) spread = most;
+  // Row groups per expert: enough workgroups to cover the CUs even with few experts, and a hot
+  // expert's long run is shared; never more than a run can use.
+  uint32_t spread = (2048 + w.E - 1) / w.E;
+  const uint64_t most = ((uint64_t)w.G * w.M + 3) / 4;
+  if (spread > most) spread = (uint32_t)most;
   if (spread > 256) spread = 256;
   if (spread < 1) spread = 1;
-  const dim3 grid(w.L * w.G, spread), block(256);
+  const dim3 grid(w.E, spread), block(256);
   if (!row_has_register_variant(w)) {
-    hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, rank, sp);
+    hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, sp);
     return (int)hipGetLastError();
   }
   const uint64_t row_bytes = (uint64_t)w.G * w.M * w.K * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
-#define PPLX_ROW_KERNEL_ARGS rank, sp, write_through
+#define PPLX_ROW_KERNEL_ARGS sp, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(split_unpack);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -317,14 +291,37 @@ int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const Disp
   return (int)hipGetLastError();
 }
 
-int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank &row,
-                              uint32_t rank, int in_dtype, void *stream) {
-  const SingleCombine tab{row};
+template <class CT>
+int launch_split_combine_send_t(const WorldDev &w, const SplitDev &sp, const CT &tab, int in_dtype,
+                                hipStream_t s) {
   const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
   const uint32_t elem_bytes = in_dtype == 0 ? 4u : 2u;
-  hipLaunchKernelGGL(split_combine_send<SingleCombine>, dim3((uint32_t)((pairs + 3) / 4)), dim3(256), 0,
-                     (hipStream_t)stream, w, tab, rank, sp, elem_bytes);
+  hipLaunchKernelGGL(split_combine_send<CT>, dim3((uint32_t)((pairs + 3) / 4)), dim3(256), 0, s, w, tab, sp,
+                     elem_bytes);
   return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                               uint32_t pick_vector, void *stream) {
+  if (pick_vector != 4 && pick_vector != 2) pick_vector = 1;
+  if (inline_rows)
+    return launch_split_dispatch_send_t(w, sp, make_inline(w, inline_rows), pick_vector, (hipStream_t)stream);
+  return launch_split_dispatch_send_t(w, sp, HbmDispatch{w.drank}, pick_vector, (hipStream_t)stream);
+}
+
+int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                               void *stream) {
+  if (inline_rows) return launch_split_dispatch_recv_t(w, sp, make_inline(w, inline_rows), (hipStream_t)stream);
+  return launch_split_dispatch_recv_t(w, sp, HbmDispatch{w.drank}, (hipStream_t)stream);
+}
+
+int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
+                              int in_dtype, void *stream) {
+  if (inline_rows)
+    return launch_split_combine_send_t(w, sp, make_inline(w, inline_rows), in_dtype, (hipStream_t)stream);
+  return launch_split_combine_send_t(w, sp, HbmCombine{w.crank}, in_dtype, (hipStream_t)stream);
 }
 
 }  // namespace pplx_amd

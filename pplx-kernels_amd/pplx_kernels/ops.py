@@ -197,7 +197,10 @@ class _World:
         # A step's kernels are enqueued by the last rank to call, so the tensors of the
         # ranks that called earlier are kept alive until then: a temporary such as
         # ``x.to(device)`` must not go back to the caching allocator before it is read.
-        self.pending: dict[str, dict[int, tuple]] = {"dispatch": {}, "combine": {}}
+        # (the same holds for every phase of split mode, which is collective as well)
+        self.pending: dict[str, dict[int, tuple]] = {
+            f"{op}{mode}": {} for op in ("dispatch", "combine") for mode in (SPLIT_NONE, SPLIT_SEND, SPLIT_RECV)
+        }
         # Widest expert_y element (bytes) that split-mode staging has been reserved for;
         # -1 = none reserved yet.
         self.split_reserved = -1
@@ -553,12 +556,11 @@ def _dispatch(
     # The library selects the world's device for the launch and restores the caller's; the
     # stream is the current one of the tensors' device (csrc/bindings/all_to_all_ops.cpp:163,194).
     check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    if mode == SPLIT_NONE:
-        world.hold(
-            "dispatch",
-            fptr,
-            (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
-        )
+    world.hold(
+        f"dispatch{mode}",
+        fptr,
+        (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
+    )
 
 
 def _combine(
@@ -580,8 +582,7 @@ def _combine(
     if mode != SPLIT_NONE:
         reserve_split(world, expert_y.element_size())
     check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    if mode == SPLIT_NONE:
-        world.hold("combine", fptr, (out_tokens, indices, weights, expert_y, bound_m))
+    world.hold(f"combine{mode}", fptr, (out_tokens, indices, weights, expert_y, bound_m))
 
 
 def _fake_dispatch(*args, **kwargs) -> None:
