@@ -190,8 +190,8 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
 //      out_expert_num_tokens.
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit,
-                                                                  uint32_t kper, uint32_t pick_vector,
-                                                                  uint32_t write_through) {
+                                                                  uint32_t kper, uint32_t tokens_per_block,
+                                                                  uint32_t pick_vector, uint32_t write_through) {
   constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
   constexpr bool kStaged = DT::kInline;
@@ -200,8 +200,6 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
     const unsigned long long *args = reinterpret_cast<const unsigned long long *>(&tab);
     for (uint32_t i = threadIdx.x; i < kTableWords; i += kFusedThreads) lds_u64[i] = args[i];
   }
-  const uint32_t waves = kFusedThreads / kWave;
-  const uint32_t tokens_per_block = waves / ksplit;
   const uint32_t own_pairs = tokens_per_block * w.K;
   unsigned long long *dst_row = lds_u64 + kTableWords;                         // [own_pairs]
   unsigned long long *dst_scale = dst_row + own_pairs;                         // [own_pairs]
@@ -464,15 +462,23 @@ template <class DT>
 int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
   const uint32_t kWaves = fused_threads((int)((w.Hb / 16 + kWave - 1) / kWave)) / kWave;
-  const uint32_t ksplit = pick_ksplit(w, kWaves);
+  // Tokens per workgroup: as few as still give every CU a workgroup (all of a workgroup's waves
+  // help with the counting; only the waves that own a token, or a share of one, load and store
+  // rows, and few storing waves per CU suit the memory system better than sixteen: 8 x 128 DSv3
+  // tokens take 14.7 us with 4 row waves per workgroup against 15.1 us with 16).  Steps of fewer
+  // than 1024 tokens spread each token's picks over several waves instead.
+  uint32_t tokens_per_block = (tokens + 255) / 256;
+  if (tokens_per_block > kWaves) tokens_per_block = kWaves;
+  if (tokens_per_block < 1) tokens_per_block = 1;
+  uint32_t ksplit = 1;
+  while (ksplit * 2 <= w.K && tokens_per_block * ksplit * 2 <= kWaves && (uint64_t)tokens * ksplit < 1024) ksplit *= 2;
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
-  const uint32_t tokens_per_block = kWaves / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
   const uint32_t lds = fused_lds_bytes(w, tokens_per_block, DT::kInline);
   // Rows that fit the last-level cache with room to spare are written through into it.
   const uint64_t row_bytes = (uint64_t)tokens * w.K * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
-#define PPLX_ROW_KERNEL_ARGS ksplit, kper, pick_vector, write_through
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper, tokens_per_block, pick_vector, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
