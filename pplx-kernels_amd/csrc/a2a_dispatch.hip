@@ -408,19 +408,23 @@ uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
 }
 
 // Scatter waves a CU should hold at a time (0 = as many as fit).
-// Measured on 8 x 4096 tokens (us at 32 = full occupancy / 3 / 4 / 6 / 8 / 12 waves per CU):
-//   59 KiB stored per wave (DSv3 fp8, top-8)   449 / 418 / 441 / 446 / 444 / 437
-//   32 KiB (bf16 2048, top-8)                  227 / 207 / 217 / 219 / 220 / 223
-//   16 KiB (bf16 4096, top-2)                  170 / 179 / 153 / 163 / 165 / 167
-//    8 KiB (bf16 512, top-8)                    65 / 126 /  79 /  64 /  60 /  61
-//    4 KiB (bf16 1024, top-2)                   46 / 110 /  71 /  59 /  53 /  49
-// A wave's loads and launch are dead time for the stores, so the less a wave stores the more
-// of them it takes to keep the CU's stores going.
+// Measured on 8 x 4096 tokens (us at 2 / 3 / 4 / 6 / 8 waves per CU / full occupancy):
+//   59 KiB stored per wave (DSv3 fp8 rows, top-8)     419 / 423 / 439 / 444 / 441 / 449
+//   32 KiB (4 KiB rows, top-8)                        210 / 213 / 217 / 220 / 221 / 227
+//   16 KiB (8 KiB rows, top-2)                        180 / 153 / 153 / 163 / 165 / 170
+//   17 KiB (2 KiB fp8 rows with scales, top-8)        178 / 137 / 119 / 110 / 111 / 117
+//    8 KiB (1 KiB rows, top-8)                        128 /  95 /  80 /  65 /  59 /  65
+//    4 KiB (2 KiB rows, top-2)                        112 /  85 /  72 /  59 /  53 /  46
+// and on the large prefill with ragged token counts and skewed routing (8 x <= 8192 DSv3 tokens):
+// 457 / 447 / 459 us at 2 / 3 / 4, 474 us at full occupancy.  A wave's loads and launch are
+// dead time for the stores, so the less a wave stores the more of them it takes to keep the
+// CU's stores going.
 uint32_t scatter_waves_per_cu(const WorldDev &w, uint32_t picks_per_wave) {
   if (w.lds_per_cu == 0) return 0;
-  const uint64_t stored = (uint64_t)picks_per_wave * (w.Hb + 4ull * w.S);
+  const uint64_t row = w.Hb + 4ull * w.S;
+  const uint64_t stored = (uint64_t)picks_per_wave * row;
   if (stored >= 24 * 1024) return 3;
-  if (stored >= 12 * 1024) return 4;
+  if (stored >= 12 * 1024) return row >= 4096 ? 4 : 6;
   if (stored >= 6 * 1024) return 8;
   return 0;
 }
@@ -437,13 +441,13 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
   const uint64_t waves = (uint64_t)tokens * ksplit;
   // One wave per workgroup, and few of them per CU at a time.  A wave reads one row and then
   // has up to K rows of stores to issue; HBM takes those stores best when a CU sends the rows of
-  // three or four waves at a time rather than those of thirty-two interleaved (measured: 8 x
-  // <= 8192 DSv3 fp8 tokens, top-8: 474 us at full occupancy, 457 / 447 / 459 us at 2 / 3 / 4
-  // waves per CU; 8 x 4096 bf16 tokens of 8 KiB, top-2: 164 us at full occupancy, 149 / 146 us
-  // at 3 / 4).  The hardware has no such knob, so each workgroup asks for a share of the CU's
-  // LDS that only that many fit into.
+  // three or four waves at a time rather than those of thirty-two interleaved (figures at
+  // scatter_waves_per_cu).  The hardware has no such knob, so each workgroup asks for a share of
+  // the CU's LDS that only that many fit into.
   const uint32_t waves_per_cu = scatter_waves_per_cu(w, kper);
-  uint32_t lds = waves_per_cu ? (w.lds_per_cu / waves_per_cu) & ~1023u : 0u;
+  // (LDS is handed out in blocks: a share that is not a multiple of 4 KiB can round up past
+  // what the intended number of workgroups leaves room for)
+  uint32_t lds = waves_per_cu ? (w.lds_per_cu / waves_per_cu) & ~4095u : 0u;
   if (lds > 65536u) lds = 65536u;
   const dim3 grid((uint32_t)waves), block(kWave);
 #define PPLX_ROW_KERNEL_ARGS ksplit, kper
