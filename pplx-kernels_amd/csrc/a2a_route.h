@@ -194,20 +194,23 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
     // Exclusive prefix of counts_out over experts: where each expert's rows start in the
     // group's compact staging area.  counts_out was written above or by route_scan.
     __syncthreads();
-    uint32_t *scan = reinterpret_cast<uint32_t *>(lds_mask);  // blockDim entries, LDS is free now
+    uint32_t *wave_total = reinterpret_cast<uint32_t *>(lds_mask);  // one entry per wave, LDS is free now
     const uint32_t per_thread = (w.E + blockDim.x - 1) / blockDim.x;
     const uint32_t e0 = threadIdx.x * per_thread;
     uint32_t local = 0;
     for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) local += span.counts_out[e];
-    scan[threadIdx.x] = local;
-    __syncthreads();
-    for (uint32_t step = 1; step < blockDim.x; step *= 2) {
-      const uint32_t add = threadIdx.x >= step ? scan[threadIdx.x - step] : 0;
-      __syncthreads();
-      scan[threadIdx.x] += add;
-      __syncthreads();
+    // prefix inside the wave by shuffles, then over the waves' totals
+    uint32_t incl = local;
+#pragma unroll
+    for (uint32_t d = 1; d < kWave; d *= 2) {
+      const uint32_t up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += up;
     }
-    uint32_t running = scan[threadIdx.x] - local;
+    if (lane == kWave - 1) wave_total[chunk] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (uint32_t i = 0; i < chunk; ++i) before += wave_total[i];
+    uint32_t running = before + incl - local;
     for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) {
       span.offsets_out[e] = running;
       running += span.counts_out[e];
