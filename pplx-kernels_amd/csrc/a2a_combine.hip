@@ -68,27 +68,30 @@ template <> struct Store8<_Float16> {
   }
 };
 
-// N picks starting at k: all N loads are issued before the first is used.
-template <typename T, int N>
-__device__ __forceinline__ void gather_group(f32x8 &acc, uint64_t row_of_lane, float weight_of_lane,
-                                             uint32_t k, uint32_t vec) {
-  typename Row8<T>::Raw raw[N];
+// N picks starting at k, VPL vectors of each: all N * VPL loads are issued before the first is used.
+template <typename T, int N, int VPL>
+__device__ __forceinline__ void gather_group(f32x8 (&acc)[VPL], uint64_t row_of_lane, float weight_of_lane,
+                                             uint32_t k, const uint32_t (&vec)[VPL]) {
+  typename Row8<T>::Raw raw[VPL][N];
 #pragma unroll
-  for (int i = 0; i < N; ++i) raw[i] = Row8<T>::load(read_lane64(row_of_lane, k + i), vec);
-  Row8<T>::template settle<N>(raw);
+  for (int v = 0; v < VPL; ++v) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) raw[v][i] = Row8<T>::load(read_lane64(row_of_lane, k + i), vec[v]);
+  }
+  Row8<T>::template settle<VPL * N>(&raw[0][0]);
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     const float wk = __builtin_bit_cast(
         float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight_of_lane), (int)(k + i)));
-    acc += wk * Row8<T>::widen(raw[i]);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) acc[v] += wk * Row8<T>::widen(raw[v][i]);
   }
 }
 
-// One wave owns VPL * 64 consecutive 8-element vectors of one output row.  With
-// KK == 0 (any K) it is one vector per lane and the picks go in groups of up to
-// eight loads; with KK in {1, 2, 4} the wave takes VPL = 8 / KK vectors per lane so
-// that eight row loads per lane are in flight for small top-k too.
-template <typename T, typename U, class CT, int KK, int VPL>
+// One wave owns VPL * 64 consecutive 8-element vectors of one output row (VPL KiB of a bf16
+// row) and takes the picks KB at a time, so KB * VPL row loads per lane are in flight: few
+// picks read long pieces of their rows, many picks shorter ones.
+template <typename T, typename U, class CT, int KB, int VPL>
 __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments,
                                                       uint32_t first_rank, uint32_t rank_count,
                                                       const uint8_t *stage_y, uint64_t stage_row_bytes) {
@@ -137,66 +140,77 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
     // A pick without a row (bad expert id or slot) contributes nothing.
     for (int v = 0; v < VPL; ++v) {
       const uint32_t vec = (segment * VPL + v) * kWave + lane;
-      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
-      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const uint32_t one[1] = {vec < nvec ? vec : nvec - 1};
+      f32x8 acc[1] = {{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}};
       for (uint32_t k = 0; k < K; ++k) {
-        if (read_lane64(row, k) != 0) gather_group<T, 1>(acc, row, weight, k, vec_ld);
+        if (read_lane64(row, k) != 0) gather_group<T, 1, 1>(acc, row, weight, k, one);
       }
-      if (vec < nvec) Store8<U>::at(out, vec, acc);
+      if (vec < nvec) Store8<U>::at(out, vec, acc[0]);
     }
     return;
   }
-  if (KK == 0) {
-    const uint32_t vec = segment * kWave + lane;
-    const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;  // clamp: loads stay unconditional
-    f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    uint32_t k = 0;
-    for (; k + 8 <= K; k += 8) gather_group<T, 8>(acc, row, weight, k, vec_ld);
-    if (K & 4) { gather_group<T, 4>(acc, row, weight, k, vec_ld); k += 4; }
-    if (K & 2) { gather_group<T, 2>(acc, row, weight, k, vec_ld); k += 2; }
-    if (K & 1) { gather_group<T, 1>(acc, row, weight, k, vec_ld); }
-    if (vec < nvec) Store8<U>::at(out, vec, acc);
-  } else {
-    constexpr int N = KK == 0 ? 1 : KK;
-    typename Row8<T>::Raw raw[VPL][N];
+  uint32_t vec_ld[VPL];
+  f32x8 acc[VPL];
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-      const uint32_t vec = (segment * VPL + v) * kWave + lane;
-      const uint32_t vec_ld = vec < nvec ? vec : nvec - 1;
-#pragma unroll
-      for (int k = 0; k < N; ++k) raw[v][k] = Row8<T>::load(read_lane64(row, k), vec_ld);
-    }
-    Row8<T>::template settle<VPL * N>(&raw[0][0]);
-#pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-      const uint32_t vec = (segment * VPL + v) * kWave + lane;
-      f32x8 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int k = 0; k < N; ++k) {
-        const float wk = __builtin_bit_cast(
-            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), k));
-        acc += wk * Row8<T>::widen(raw[v][k]);
-      }
-      if (vec < nvec) Store8<U>::at(out, vec, acc);
-    }
+  for (int v = 0; v < VPL; ++v) {
+    const uint32_t vec = (segment * VPL + v) * kWave + lane;
+    vec_ld[v] = vec < nvec ? vec : nvec - 1;  // clamp: loads stay unconditional
+    acc[v] = f32x8{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   }
+  uint32_t k = 0;
+  for (; k + KB <= K; k += KB) gather_group<T, KB, VPL>(acc, row, weight, k, vec_ld);
+  if constexpr (KB > 4) {
+    if ((K - k) & 4) { gather_group<T, 4, VPL>(acc, row, weight, k, vec_ld); k += 4; }
+  }
+  if constexpr (KB > 2) {
+    if ((K - k) & 2) { gather_group<T, 2, VPL>(acc, row, weight, k, vec_ld); k += 2; }
+  }
+  if constexpr (KB > 1) {
+    if ((K - k) & 1) { gather_group<T, 1, VPL>(acc, row, weight, k, vec_ld); }
+  }
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const uint32_t vec = (segment * VPL + v) * kWave + lane;
+    if (vec < nvec) Store8<U>::at(out, vec, acc[v]);
+  }
+}
+
+template <typename T, typename U, class CT, int KB, int VPL>
+int launch_combine_v(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
+                     const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
+  const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
+  const uint32_t segments = (nvec_segments + VPL - 1) / VPL;
+  const uint64_t waves = (uint64_t)rank_count * w.M * segments;
+  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
+  hipLaunchKernelGGL((combine_gather<T, U, CT, KB, VPL>), grid, block, 0, s, w, tab, segments, first_rank,
+                     rank_count, stage_y, stage_row_bytes);
+  return (int)hipGetLastError();
 }
 
 template <typename T, typename U, class CT>
 int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
                      const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
+#define PPLX_COMBINE(KB, VPL) \
+  return launch_combine_v<T, U, CT, KB, VPL>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s)
+  // Few picks: long pieces of each row, all picks at once.  Many picks: all of them at once,
+  // 1 KiB of each (eight loads per lane in flight either way) -- except for steps of a few
+  // hundred to two thousand tokens, whose waves are all resident at the same moment: there the
+  // picks are better taken one after the other in 7 or 8 KiB pieces by a quarter as many waves
+  // (8 x 128 DSv3 tokens, top-8: 23.4 us against 25.3 us; 8 x 256: 45.8 against 46.8; from
+  // 8 x 512 on the wide form wins, 88.7 against 91.5 us, and below 8 x 64 too).
   const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
-  const uint32_t vpl = w.K == 1 ? 8 : w.K == 2 ? 4 : w.K == 4 ? 2 : 1;
-  const uint32_t segments = (nvec_segments + vpl - 1) / vpl;
-  const uint64_t waves = (uint64_t)rank_count * w.M * segments;
-  const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
-  switch (w.K) {
-    case 1: hipLaunchKernelGGL((combine_gather<T, U, CT, 1, 8>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
-    case 2: hipLaunchKernelGGL((combine_gather<T, U, CT, 2, 4>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
-    case 4: hipLaunchKernelGGL((combine_gather<T, U, CT, 4, 2>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
-    default: hipLaunchKernelGGL((combine_gather<T, U, CT, 0, 1>), grid, block, 0, s, w, tab, segments, first_rank, rank_count, stage_y, stage_row_bytes); break;
+  const uint64_t tokens = (uint64_t)rank_count * w.M;
+  if (w.K > 4 && tokens > 384 && tokens <= 2048 && nvec_segments >= 7) {
+    if (nvec_segments % 7 == 0) PPLX_COMBINE(1, 7);
+    PPLX_COMBINE(1, 8);
   }
-  return (int)hipGetLastError();
+  switch (w.K) {
+    case 1: PPLX_COMBINE(1, 8);
+    case 2: PPLX_COMBINE(2, 4);
+    case 4: PPLX_COMBINE(4, 2);
+    default: PPLX_COMBINE(8, 1);
+  }
+#undef PPLX_COMBINE
 }
 
 template <class CT>

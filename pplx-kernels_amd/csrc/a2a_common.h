@@ -110,9 +110,18 @@ __device__ __forceinline__ void settle(V &v) {
 
 // settle() for N registers at once: every load feeding them has to be issued
 // before this point, so the N loads go out back to back behind one wait.
-template <int N> struct SettleAll;
+template <int N> struct SettleAll {
+  // other counts: in pieces of 8, 4, 2, 1 (the common counts below are one statement each)
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    constexpr int kHead = N >= 8 ? 8 : N >= 4 ? 4 : N >= 2 ? 2 : 1;
+    SettleAll<kHead>::of(r);
+    if constexpr (N > kHead) SettleAll<N - kHead>::of(r + kHead);
+  }
+};
 template <> struct SettleAll<1> {
-  template <typename V> static __device__ __forceinline__ void of(V *r) { asm volatile("" : "+v"(r[0])); }
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]));
+  }
 };
 template <> struct SettleAll<2> {
   template <typename V> static __device__ __forceinline__ void of(V *r) {
@@ -124,19 +133,24 @@ template <> struct SettleAll<4> {
     asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
   }
 };
+template <> struct SettleAll<7> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]));
+  }
+};
 template <> struct SettleAll<8> {
   template <typename V> static __device__ __forceinline__ void of(V *r) {
-    asm volatile(""
-                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
-                   "+v"(r[7]));
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+  }
+};
+template <> struct SettleAll<14> {
+  template <typename V> static __device__ __forceinline__ void of(V *r) {
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]));
   }
 };
 template <> struct SettleAll<16> {
   template <typename V> static __device__ __forceinline__ void of(V *r) {
-    asm volatile(""
-                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]),
-                   "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]),
-                   "+v"(r[13]), "+v"(r[14]), "+v"(r[15]));
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]), "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]), "+v"(r[15]));
   }
 };
 

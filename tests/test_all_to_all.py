@@ -410,6 +410,28 @@ def test_combine_dtype_matrix(y_dtype, out_dtype):
 
 
 @pytest.mark.parametrize(
+    "hidden,y_dtype,out_dtype",
+    [
+        (7168, torch.float16, torch.bfloat16),
+        (4096, torch.float32, torch.float16),
+        (3600, torch.bfloat16, torch.bfloat16),  # the last 1 KiB piece of a row is partial
+        (8192 + 512, torch.bfloat16, torch.float16),
+    ],
+)
+def test_combine_of_mid_size_steps(hidden, y_dtype, out_dtype):
+    """Steps of a few hundred to two thousand tokens with more than four picks take the combine
+    variant that reads one pick at a time in 7 or 8 KiB pieces."""
+    spec = _small_spec(
+        name=f"mid{hidden}", world_size=4, num_experts=32, experts_per_token=6, max_num_tokens=130,
+        hidden_dim=hidden, expert_y_dtype=y_dtype, out_dtype=out_dtype, tokens="uniform",
+    )  # fmt: skip
+    groups = generate(spec)
+    groups[0].n = spec.max_num_tokens
+    groups[1].n = 0
+    run_and_check(spec, groups, use_numpy=True)
+
+
+@pytest.mark.parametrize(
     "E,K,M,R",
     [
         (512, 8, 300, 8), (1024, 4, 130, 4), (8, 8, 70, 2), (4, 1, 5, 1), (64, 6, 1500, 2), (2048, 2, 40, 2),
@@ -637,6 +659,8 @@ def _combine_kw(step, r):
         dict(name="split-10k-row", hidden_dim=5120, max_num_tokens=6),
         dict(name="split-14k-row", hidden_dim=7168, max_num_tokens=6),
         dict(name="split-f32y", expert_y_dtype=torch.float32, out_dtype=torch.float16),
+        # a step of a few hundred tokens, top-6: combine RECV takes its picks one at a time
+        dict(name="split-mid", max_num_tokens=128, experts_per_token=6, hidden_dim=7168),
     ],
     ids=lambda kw: kw["name"],
 )
