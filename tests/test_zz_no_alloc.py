@@ -160,3 +160,58 @@ def test_static_step_reports_faults_and_refuses_what_does_not_fit():
     assert lib.pplx_a2a_static_step(ctypes.byref(wide), 0, d_args, None, None, stream) == 4
     assert lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, None, None, None, stream) == 1
     assert lib.pplx_a2a_static_step(None, 0, d_args, None, None, stream) == 1
+
+
+def test_static_step_replays_from_a_graph():
+    """One of the callers the entry point is for: a step recorded into a hipGraph without any
+    world.  The first call on a device looks up the library's scratch array and is made eagerly;
+    the recorded one is replayed with new inputs and compared with the world path each time."""
+    from pplx_kernels import ops
+
+    lib = ops.load_library()
+    spec = _spec(name="graph", world_size=4, num_experts=32, experts_per_token=8, hidden_dim=512,
+                 max_num_tokens=40)  # fmt: skip
+    groups = generate(spec)
+    got = _zeroed_step(spec, groups, None)
+    ref = _zeroed_step(spec, groups, None)
+    cfg = _config(ops, spec)
+    d_args, c_args = _pack(ops, spec, got)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        ops.check_status(lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, d_args, c_args, None, stream.cuda_stream))
+        stream.synchronize()
+        graph = ctypes.c_void_p()
+        ops.check_status(lib.pplx_a2a_graph_begin_capture(stream.cuda_stream))
+        ops.check_status(lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, d_args, c_args, None, stream.cuda_stream))
+        ops.check_status(lib.pplx_a2a_graph_end_capture(stream.cuda_stream, ctypes.byref(graph)))
+    world = make_world(spec, group_name="static-graph-ref")
+    for replay in range(3):
+        fresh = generate(spec, seed=20 + replay)
+        for step in (got, ref):
+            for r in range(spec.world_size):
+                g = fresh[r // spec.dp_size]
+                step.dp_x[r].copy_(g.x)
+                step.dp_x_scale[r].copy_(g.x_scale)
+                step.indices[r].copy_(g.indices.to(torch.uint32))
+                step.weights[r].copy_(g.weights)
+                step.bound_m[r].fill_(g.n)
+                step.out_tokens[r].fill_(float("nan"))
+            step.expert_x_all.view(torch.uint8).zero_()
+            step.expert_x_scale_all.zero_()
+            step.expert_y_all.copy_(torch.randn(step.expert_y_all.shape, generator=torch.Generator(device="cuda").manual_seed(replay), device="cuda"))
+        torch.cuda.synchronize()
+        ref.dispatch_world(world)
+        ref.combine_world(world)
+        ops.check_status(lib.pplx_a2a_graph_launch(graph, stream.cuda_stream))
+        stream.synchronize()
+        torch.cuda.synchronize()
+        assert torch.equal(got.expert_num_tokens_all, ref.expert_num_tokens_all)
+        assert int(ref.expert_num_tokens_all.sum()) == spec.experts_per_token * sum(g.n for g in fresh)
+        assert torch.equal(got.expert_x_all.view(torch.uint8), ref.expert_x_all.view(torch.uint8))
+        assert torch.equal(got.expert_x_scale_all.view(torch.int32), ref.expert_x_scale_all.view(torch.int32))
+        for r in range(spec.world_size):
+            n = fresh[r // spec.dp_size].n
+            assert torch.equal(got.out_tokens[r][:n].view(torch.int16), ref.out_tokens[r][:n].view(torch.int16))
+    ops.check_status(lib.pplx_a2a_graph_destroy(graph))
+    assert world.faults() == 0
+    world.destroy()
