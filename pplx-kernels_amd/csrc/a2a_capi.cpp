@@ -840,6 +840,19 @@ int pplx_a2a_destroy(pplx_a2a_t *h) {
       w.arrived_combine[h->rank] = 0;
       --w.n_arrived_combine;
     }
+    // ... and the same for a phase of split mode that has not been launched yet
+    if (w.split_ready) {
+      auto forget = [&](std::vector<uint8_t> &made, uint32_t &count) {
+        if (count < w.dev.R && made[h->rank]) {
+          made[h->rank] = 0;
+          --count;
+        }
+      };
+      forget(w.dsend, w.n_dsend);
+      forget(w.drecv, w.n_drecv);
+      forget(w.csend, w.n_csend);
+      forget(w.crecv, w.n_crecv);
+    }
   }
   delete h;
   return PPLX_A2A_OK;

@@ -383,6 +383,30 @@ def test_first_split_step_is_capturable_once_reserved():
         a.destroy()
 
 
+def test_a_rank_replaced_in_the_middle_of_a_split_phase():
+    """A handle destroyed after its SEND call, before the phase is complete, takes that call with
+    it: the handle that replaces it sends again and the step comes out whole."""
+    from pplx_kernels import AllToAll
+
+    spec = _spec(name="split-replace", in_dtype=FP8, hidden_dim=512)
+    step = DeviceStep(spec, generate(spec))
+    ranks = _make_ranks(spec, "split-replace")
+    R = spec.world_size
+    ranks[1].dispatch(**_dispatch_kw(step, 1), do_send=True, do_recv=False)
+    ranks[1].destroy()
+    ranks[1] = AllToAll.intranode(
+        spec.max_num_tokens, spec.num_experts, spec.experts_per_token, 1, spec.world_size, spec.dp_size,
+        spec.hidden_dim, spec.hidden_dim_bytes, spec.hidden_dim_scale_bytes, group_name="split-replace",
+    )  # fmt: skip
+    for r in range(R):
+        ranks[r].dispatch(**_dispatch_kw(step, r), do_send=True, do_recv=False)
+    for r in range(R):
+        ranks[r].dispatch(**_dispatch_kw(step, r), do_send=False, do_recv=True)
+    check_dispatch_against_oracle(step)
+    for a in ranks:
+        a.destroy()
+
+
 # ---------------------------------------------------------------------------
 # Many routing tiles (the prefix over tiles takes several trips)
 # ---------------------------------------------------------------------------
