@@ -477,14 +477,9 @@ int run_combine(pplx_a2a_world &w, void *stream) {
   return PPLX_A2A_OK;
 }
 
-uint64_t round_up(uint64_t x, uint64_t to) { return (x + to - 1) / to * to; }
-
 void free_split(pplx_a2a_world &w) {
   SplitDev &sp = w.split;
-  (void)hipFree(sp.stage_x);
-  (void)hipFree(sp.gexp);
-  (void)hipFree(sp.gcnt);
-  (void)hipFree(sp.goff);
+  (void)hipFree(sp.stage_x);  // gexp and gcnt live behind the rows
   (void)hipFree(sp.stage_y);
   sp = SplitDev{};
   w.split_ready = false;
@@ -503,25 +498,17 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
   if (!w.split_ready) {
     if (w.n_arrived_dispatch != 0 || w.n_arrived_combine != 0)
       return fail(PPLX_A2A_INVALID_STATE, "a step is being assembled");
-    sp.token_stride = (uint32_t)round_up((uint64_t)d.Hb + 4ull * d.S + 4, 16);
-    struct Alloc {
-      void **ptr;
-      size_t bytes;
-    } allocs[] = {
-        {reinterpret_cast<void **>(&sp.stage_x), pairs * sp.token_stride},
-        {reinterpret_cast<void **>(&sp.gexp), sizeof(uint32_t) * pairs},
-        {reinterpret_cast<void **>(&sp.gcnt), sizeof(uint32_t) * (size_t)d.E},
-        {reinterpret_cast<void **>(&sp.goff), sizeof(uint32_t) * (size_t)d.E},
-    };
-    for (const Alloc &a : allocs) {
-      hipError_t err = hipMalloc(a.ptr, a.bytes);
-      if (err == hipSuccess) err = hipMemset(*a.ptr, 0, a.bytes);
-      if (err != hipSuccess) {
-        free_split(w);
-        return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of split-mode staging failed: %s", a.bytes,
-                    hipGetErrorString(err));
-      }
+    const StageLayout lay = stage_layout(d.Hb, d.S, pairs, d.E);
+    hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_x), lay.bytes);
+    if (err == hipSuccess) err = hipMemset(sp.stage_x, 0, lay.bytes);
+    if (err != hipSuccess) {
+      free_split(w);
+      return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of split-mode staging failed: %s", (size_t)lay.bytes,
+                  hipGetErrorString(err));
     }
+    sp.token_stride = lay.token_stride;
+    sp.gexp = reinterpret_cast<uint32_t *>(sp.stage_x + lay.gexp_offset);
+    sp.gcnt = reinterpret_cast<uint32_t *>(sp.stage_x + lay.gcnt_offset);
     w.dsend.assign(d.R, 0);
     w.drecv.assign(d.R, 0);
     w.csend.assign(d.R, 0);

@@ -197,10 +197,11 @@ int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint
   // hundred to two thousand tokens, whose waves are all resident at the same moment: there the
   // picks are better taken one after the other in 7 or 8 KiB pieces by a quarter as many waves
   // (8 x 128 DSv3 tokens, top-8: 23.4 us against 25.3 us; 8 x 256: 45.8 against 46.8; from
-  // 8 x 512 on the wide form wins, 88.7 against 91.5 us, and below 8 x 64 too).
+  // 8 x 512 on the wide form wins, 88.7 against 91.5 us, and below 8 x 64 too).  Staged rows
+  // (the K rows of a token lie side by side) stay with the wide form: 24 us against 32 us.
   const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
   const uint64_t tokens = (uint64_t)rank_count * w.M;
-  if (w.K > 4 && tokens > 384 && tokens <= 2048 && nvec_segments >= 7) {
+  if (!CT::kStaged && w.K > 4 && tokens > 384 && tokens <= 2048 && nvec_segments >= 7) {
     if (nvec_segments % 7 == 0) PPLX_COMBINE(1, 7);
     PPLX_COMBINE(1, 8);
   }

@@ -91,27 +91,44 @@ struct RouteSpan {
   uint32_t *tile_cnt;     // [tiles][E]
   uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
   // split mode only:
-  uint32_t *expert_out;   // [G * M][K] expert of every pair
+  uint32_t *expert_out;   // [G * M][K] expert of every pair (num_experts = the pair has no row)
   uint32_t *counts_out;   // [E] rows per expert
-  uint32_t *offsets_out;  // [E] exclusive prefix of counts_out over experts
 };
 
 // Device state of split send / recv mode: a two-hop path through staging that the world
-// owns.  dispatch SEND packs every routed row, grouped by expert and ordered by slot, into
-// stage_x in the reference's wire format  row | fp32 scales | u32 source token, padded to 16
-// bytes (csrc/all_to_all/intranode.cpp:41-47, csrc/all_to_all/intranode_dispatch.cu:60-61,148-150);
-// dispatch RECV unpacks into the callers' expert-major outputs.  combine SEND copies expert
-// rows into stage_y, one row per (token, pick); combine RECV reduces them.
+// owns.  dispatch SEND routes the step and leaves one copy of the row per (token, pick) in
+// stage_x, in the order of the picks, in the reference's wire format  row | fp32 scales | u32
+// source token, padded to 16 bytes (csrc/all_to_all/intranode.cpp:41-47,
+// csrc/all_to_all/intranode_dispatch.cu:60-61,148-150); dispatch RECV moves each staged row to
+// its slot in the callers' expert-major outputs.  combine SEND copies expert rows into stage_y,
+// one row per (token, pick); combine RECV reduces them.
 struct SplitDev {
-  uint8_t *stage_x;        // [G * M * K rows][token_stride], expert e's rows start at goff[e]
+  uint8_t *stage_x;        // [G * M][K][token_stride]
   uint32_t token_stride;   // round_up(Hb + 4 S + 4, 16)
   uint32_t pad_;
   uint32_t *gexp;          // [G * M][K] expert of a pair (num_experts = the pair has no row)
   uint32_t *gcnt;          // [E] rows sent to expert e
-  uint32_t *goff;          // [E] exclusive prefix of gcnt over the experts
   uint8_t *stage_y;        // [G * M * K][y_row_bytes]
   uint64_t y_row_bytes;
 };
+
+// stage_x, gexp and gcnt are one allocation, in this order, so that a kernel short of scalar
+// registers can take the first pointer alone and work out the rest.
+struct StageLayout {
+  uint32_t token_stride;
+  uint64_t gexp_offset, gcnt_offset, bytes;
+};
+#ifdef __HIPCC__
+__host__ __device__
+#endif
+inline StageLayout stage_layout(uint32_t row_bytes, uint32_t scales, uint64_t pairs, uint32_t experts) {
+  StageLayout l;
+  l.token_stride = (row_bytes + 4u * scales + 4u + 15u) & ~15u;
+  l.gexp_offset = pairs * l.token_stride;
+  l.gcnt_offset = l.gexp_offset + pairs * 4u;
+  l.bytes = l.gcnt_offset + 4ull * experts;
+  return l;
+}
 
 // Worlds of up to kInlineRanks ranks pass their rank tables to the kernels as
 // kernel arguments (9 KiB for dispatch, 5 KiB for combine; HIP on gfx950 takes kernel
@@ -156,7 +173,9 @@ int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t
                     void *stream);
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
-// Split mode phases, each for all ranks at once (`inline_rows` as above).
+// Split mode phases, each for all ranks at once (`inline_rows` as above).  launch_split_pack is
+// the second half of a dispatch SEND whose routing ran as launches of its own.
+int launch_split_pack(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows, void *stream);
 int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
                                uint32_t pick_vector, void *stream);
 int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,

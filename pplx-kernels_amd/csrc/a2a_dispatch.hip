@@ -188,10 +188,14 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
 //      destination rows once for the workgroup and leave them in LDS;
 //   4. the waves fan their rows out.  The last workgroup has counted everything and writes
 //      out_expert_num_tokens.
+// As dispatch SEND of split mode (`stage` = SplitDev::stage_x) the launch leaves the callers'
+// outputs alone: the row of pair (token, pick) goes to the pair's staging row, its expert and
+// the rows per expert to the tables behind the rows (stage_layout).
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit,
                                                                   uint32_t kper, uint32_t tokens_per_block,
-                                                                  uint32_t pick_vector, uint32_t write_through) {
+                                                                  uint32_t pick_vector, uint32_t write_through,
+                                                                  uint8_t *stage) {
   constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
   constexpr bool kStaged = DT::kInline;
@@ -298,9 +302,25 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   }
   if (threadIdx.x < own_pairs) {
     Destination d;
-    if (pick_live) {
+    const size_t pair = (size_t)pick_v * w.K + pick_k;
+    if (stage != nullptr) {
+      // (whether the slot fits the receiver's rows is for RECV to say)
+      const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
+      const bool has_row = pick_live && pick_e < w.E && pick_slot != kInvalidSlot;
+      if (has_row) {
+        d.row = reinterpret_cast<uint64_t>(stage + pair * lay.token_stride);
+        d.scale = d.row + w.Hb;
+        d.scale_step = 1;
+        *global_ptr<uint32_t>(d.row + w.Hb + 4ull * w.S) = pick_t;
+      }
+      if (pick_v < total) {
+        as_global(reinterpret_cast<uint32_t *>(stage + lay.gexp_offset))[pair] = has_row ? pick_e : w.E;
+      }
+    } else if (pick_live) {
       d = resolve_destination(w, rows(), pick_e, pick_slot, true);
-      as_global(w.slot_map)[(size_t)pick_v * w.K + pick_k] = pick_slot;
+    }
+    if (pick_live) {
+      as_global(w.slot_map)[pair] = pick_slot;
       if (pick_e >= w.E) {
         atomicOr(w.faults, kFaultBadExpert);
       } else if (pick_repeats) {
@@ -314,6 +334,11 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   __syncthreads();
   if (blockIdx.x == gridDim.x - 1) {
     for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) {
+      if (stage != nullptr) {
+        const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
+        as_global(reinterpret_cast<uint32_t *>(stage + lay.gcnt_offset))[e] = hist[e];
+        continue;
+      }
       const DispatchRank &owner = rows().at(e / w.L);
       as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
     }
@@ -463,7 +488,8 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
 }
 
 template <class DT>
-int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
+int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s,
+                   uint8_t *stage = nullptr) {
   const uint32_t tokens = w.G * w.M;
   const uint32_t kWaves = fused_threads((int)((w.Hb / 16 + kWave - 1) / kWave)) / kWave;
   // Tokens per workgroup: as few as still give every CU a workgroup (all of a workgroup's waves
@@ -482,7 +508,7 @@ int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipSt
   // Rows that fit the last-level cache with room to spare are written through into it.
   const uint64_t row_bytes = (uint64_t)tokens * w.K * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
-#define PPLX_ROW_KERNEL_ARGS ksplit, kper, tokens_per_block, pick_vector, write_through
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper, tokens_per_block, pick_vector, write_through, stage
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -511,9 +537,7 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hi
 // Launchers
 // ---------------------------------------------------------------------------
 uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
-  const uint32_t tables = tile_chunks * num_experts * (uint32_t)(sizeof(unsigned long long) + sizeof(uint32_t));
-  const uint32_t scan = tile_chunks * kWave * (uint32_t)sizeof(uint32_t);  // split mode's block scan
-  return tables > scan ? tables : scan;
+  return tile_chunks * num_experts * (uint32_t)(sizeof(unsigned long long) + sizeof(uint32_t));
 }
 
 bool dispatch_is_fused(const WorldDev &w) {
@@ -537,6 +561,34 @@ int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stre
   hipLaunchKernelGGL((bind_rows<BindCombineBatch, CombineRank>), dim3(1), dim3(256), 0,
                      (hipStream_t)stream, w.crank, b);
   return (int)hipGetLastError();
+}
+
+// dispatch SEND of split mode: the routing of the one-call form, rows into the staging area.
+template <class DT>
+int launch_split_dispatch_send_t(const WorldDev &w, const SplitDev &sp, const DT &tab, uint32_t pick_vector,
+                                 const DispatchRank *inline_rows, hipStream_t s) {
+  if (dispatch_is_fused(w)) return launch_fused_t(w, tab, pick_vector, s, sp.stage_x);
+  RouteSpan span{};
+  span.v_begin = 0;
+  span.v_count = w.G * w.M;
+  span.tile_chunks = w.tile_chunks;
+  span.pick_vector = pick_vector;
+  span.tile_cnt = w.tile_cnt;
+  span.slot_out = w.slot_map;
+  span.expert_out = sp.gexp;
+  span.counts_out = sp.gcnt;
+  int err = launch_route_t<DT, true>(w, tab, span, s);
+  if (err) return err;
+  return launch_split_pack(w, sp, inline_rows, s);
+}
+
+int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                               uint32_t pick_vector, void *stream) {
+  if (pick_vector != 4 && pick_vector != 2) pick_vector = 1;
+  if (inline_rows)
+    return launch_split_dispatch_send_t(w, sp, make_inline(w, inline_rows), pick_vector, inline_rows,
+                                        (hipStream_t)stream);
+  return launch_split_dispatch_send_t(w, sp, HbmDispatch{w.drank}, pick_vector, nullptr, (hipStream_t)stream);
 }
 
 int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t pick_vector, void *stream) {

@@ -22,8 +22,8 @@ namespace {
 //
 // SPLIT = false: the launch writes out_expert_num_tokens of the owning ranks.  SPLIT = true
 // (dispatch SEND of split mode, which may not touch the outputs yet): the rows per expert go to
-// counts_out instead, together with their exclusive prefix over the experts and the expert of
-// every pair, for the pack / unpack phases.
+// counts_out instead, and the expert of every pair of the span (num_experts where the pair has
+// no row) to expert_out, for the later phases.
 // ---------------------------------------------------------------------------
 
 // The token of this thread: which group and sender, whether its row of picks exists, and the
@@ -185,36 +185,12 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
       return 0u;
     });
     if (no_row.codes) atomicOr(w.faults, no_row.codes);
+  } else if (SPLIT && tok.in_span) {
+    // a token that is not there this step: none of its pairs has a row
+    for (uint32_t k = 0; k < w.K; ++k) span.expert_out[(size_t)tok.v * w.K + k] = w.E;
   }
   if (tok.in_span && tok.t == 0 && dispatch_group_overflows(w, tab, tok.g)) {
     atomicOr(w.faults, kFaultTooManyTokens);
-  }
-
-  if (SPLIT && blockIdx.x == gridDim.x - 1) {
-    // Exclusive prefix of counts_out over experts: where each expert's rows start in the
-    // group's compact staging area.  counts_out was written above or by route_scan.
-    __syncthreads();
-    uint32_t *wave_total = reinterpret_cast<uint32_t *>(lds_mask);  // one entry per wave, LDS is free now
-    const uint32_t per_thread = (w.E + blockDim.x - 1) / blockDim.x;
-    const uint32_t e0 = threadIdx.x * per_thread;
-    uint32_t local = 0;
-    for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) local += span.counts_out[e];
-    // prefix inside the wave by shuffles, then over the waves' totals
-    uint32_t incl = local;
-#pragma unroll
-    for (uint32_t d = 1; d < kWave; d *= 2) {
-      const uint32_t up = __shfl_up(incl, d, kWave);
-      if (lane >= d) incl += up;
-    }
-    if (lane == kWave - 1) wave_total[chunk] = incl;
-    __syncthreads();
-    uint32_t before = 0;
-    for (uint32_t i = 0; i < chunk; ++i) before += wave_total[i];
-    uint32_t running = before + incl - local;
-    for (uint32_t e = e0; e < e0 + per_thread && e < w.E; ++e) {
-      span.offsets_out[e] = running;
-      running += span.counts_out[e];
-    }
   }
 }
 

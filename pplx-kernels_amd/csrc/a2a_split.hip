@@ -5,10 +5,12 @@
 // csrc/all_to_all/bench_all_to_all.cpp:183-203).  In the loopback every phase is collective:
 // the ranks' calls of a phase are recorded, and the call of the last rank enqueues ONE launch
 // sequence for all of them, as in send+recv mode.
-//   dispatch SEND   routes the whole step (slot map, rows per expert and their prefix over the
-//                   experts) and packs every routed row into the staging area, grouped by
-//                   expert and ordered by slot: the expert-major receive buffer
-//   dispatch RECV   unpacks each expert's run of staged rows into the owning rank's outputs
+//   dispatch SEND   routes the whole step (slot map, rows per expert, expert of every pair) and
+//                   leaves one copy of the row per (token, pick) in the staging area, in the
+//                   order of the picks: small steps in the one launch of the one-call form
+//                   (dispatch_fused with its rows pointed at the staging area, a2a_dispatch.hip),
+//                   larger ones as the routing launches followed by split_pack
+//   dispatch RECV   moves every staged row to its slot in the owning rank's outputs
 //   combine SEND    copies the expert_y row of every (token, pick) into the pair's staging row
 //                   (the reference copies it into the source rank's inbox,
 //                   csrc/all_to_all/intranode_combine.cu:77-111)
@@ -19,14 +21,14 @@
 namespace pplx_amd {
 namespace {
 
-__device__ __forceinline__ uint8_t *stage_row(const SplitDev &sp, uint64_t position) {
-  return sp.stage_x + position * sp.token_stride;
+__device__ __forceinline__ uint8_t *stage_row(const SplitDev &sp, uint64_t pair) {
+  return sp.stage_x + pair * sp.token_stride;
 }
 
 // dispatch SEND, second half: one wave per token packs row | scales | source token for each of
 // its picks.  Lane k resolves pick k.
 template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev sp) {
+__global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev sp, uint32_t write_through) {
   const uint32_t lane = lane_id();
   const uint32_t v = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
   const uint32_t g = v / w.M;
@@ -52,26 +54,30 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev s
   uint64_t dst = 0;
   if (lane < w.K) {
     const size_t pair = (size_t)v * w.K + lane;
-    const uint32_t e = as_global(sp.gexp)[pair];
-    const uint32_t slot = as_global(w.slot_map)[pair];
-    if (e < w.E && slot != kInvalidSlot) {
-      dst = reinterpret_cast<uint64_t>(stage_row(sp, (uint64_t)as_global(sp.goff)[e] + slot));
-    }
+    if (as_global(sp.gexp)[pair] < w.E) dst = reinterpret_cast<uint64_t>(stage_row(sp, pair));
   }
 #pragma unroll
   for (int i = 0; i < NV; ++i) settle(x[i]);
   settle(sc);
   settle(dst);
-  // The staged rows are read back by the RECV phase next: they are stored write-through so
-  // that they stay in the last-level cache when they fit there.
+  // The staged rows are read back by the RECV phase next: while they fit the last-level cache
+  // they are stored write-through so that they stay there.
   for (uint32_t k = 0; k < w.K; ++k) {
     const uint64_t p = read_lane64(dst, k);
     if (p == 0) continue;
     PPLX_GLOBAL u32x4 *out = global_ptr<u32x4>(p);
+    if (write_through) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const uint32_t j = lane + i * kWave;
-      if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[i], out + j);
+      for (int i = 0; i < NV; ++i) {
+        const uint32_t j = lane + i * kWave;
+        if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[i], out + j);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const uint32_t j = lane + i * kWave;
+        if (EXACT || j < nvec) row_store<RowStore::kStreamThrough>(x[i], out + j);
+      }
     }
     PPLX_GLOBAL float *sout = global_ptr<float>(p + w.Hb);
     if (lane < S) row_store<RowStore::kKeep>(sc, sout + lane);
@@ -95,10 +101,8 @@ __global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, Split
   const PPLX_GLOBAL float *srow = as_global(src.dp_xs) + (int64_t)t * src.dp_xs_stride_row;
   for (uint32_t k = 0; k < w.K; ++k) {
     const size_t pair = (size_t)v * w.K + k;
-    const uint32_t e = as_global(sp.gexp)[pair];
-    const uint32_t slot = as_global(w.slot_map)[pair];
-    if (e >= w.E || slot == kInvalidSlot) continue;
-    uint8_t *p = stage_row(sp, (uint64_t)as_global(sp.goff)[e] + slot);
+    if (as_global(sp.gexp)[pair] >= w.E) continue;
+    uint8_t *p = stage_row(sp, pair);
     PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(p));
     for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
     PPLX_GLOBAL float *sout = as_global(reinterpret_cast<float *>(p + w.Hb));
@@ -107,91 +111,101 @@ __global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, Split
   }
 }
 
-// dispatch RECV: workgroup column blockIdx.x takes expert e; its run of staged rows goes to
-// out_expert_x / out_expert_x_scale of the owning rank, slot by slot; blockIdx.y spreads long
-// runs over workgroups.  The expert's count goes to out_expert_num_tokens.
-template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, SplitDev sp, uint32_t write_through) {
-  const uint32_t lane = lane_id();
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const uint32_t e = blockIdx.x;
-  const uint32_t el = e % w.L;
-  const DispatchRank &dst = tab.at(e / w.L);
-  const uint32_t count = as_global(sp.gcnt)[e], offset = as_global(sp.goff)[e];
-  if (blockIdx.y == 0 && threadIdx.x == 0) {
-    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)count;
-  }
-  const uint32_t nvec = w.Hb / 16;
-  const uint32_t S = w.S;
-  const uint32_t waves = blockDim.x / kWave;
-  for (uint32_t slot = blockIdx.y * waves + wave; slot < count; slot += gridDim.y * waves) {
-    if (slot >= dst.x_rows) {
-      if (lane == 0) atomicOr(w.faults, kFaultRowDropped);
-      continue;
-    }
-    const uint8_t *src = stage_row(sp, (uint64_t)offset + slot);
-    const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
-    PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
-        dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
-    u32x4 x[NV];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      uint32_t j = lane + v * kWave;
-      if (!EXACT) j = j < nvec ? j : nvec - 1;
-      x[v] = row[j];
-    }
-    float sc = 0.f;
-    const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
-    if (S) sc = sin[lane < S ? lane : S - 1];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) settle(x[v]);
-    settle(sc);
-    PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
-                              (int64_t)slot * dst.xs_stride_row;
-    // same policy as the one-call dispatch: rows that fit the last-level cache stay there
-    if (write_through) {
-#pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const uint32_t j = lane + v * kWave;
-        if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[v], out + j);
-      }
-    } else {
-#pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const uint32_t j = lane + v * kWave;
-        if (EXACT || j < nvec) row_store<RowStore::kStreamThrough>(x[v], out + j);
-      }
-    }
-    if (lane < S) row_store<RowStore::kKeep>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
-    for (uint32_t j = lane + kWave; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
+// The first workgroup of a RECV launch hands the rows per expert to the owning ranks.
+template <class DT>
+__device__ __forceinline__ void publish_counts(const WorldDev &w, const DT &tab, const SplitDev &sp) {
+  if (blockIdx.x != 0) return;
+  for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
+    const DispatchRank &dst = tab.at(e / w.L);
+    as_global(dst.out_num_tokens)[(int64_t)(e % w.L) * dst.out_num_tokens_stride] = (int32_t)as_global(sp.gcnt)[e];
   }
 }
 
+// dispatch RECV: one wave per (token, pick) moves the pair's staged row to its slot in
+// out_expert_x / out_expert_x_scale of the rank that owns the expert.  `eager`: the row is
+// fetched together with the pair's expert and slot instead of behind them (one trip to memory
+// instead of two; pays while few pairs are empty).
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, SplitDev sp, uint32_t write_through,
+                                                    uint32_t eager) {
+  publish_counts(w, tab, sp);
+  const uint32_t lane = lane_id();
+  const uint64_t pair = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
+  if (pair >= (uint64_t)w.G * w.M * w.K) return;
+  const uint32_t e = as_global(sp.gexp)[pair];
+  const uint32_t slot = as_global(w.slot_map)[pair];
+  if (!eager && (e >= w.E || slot == kInvalidSlot)) return;
+  const uint8_t *src = stage_row(sp, pair);
+  const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
+  const uint32_t nvec = w.Hb / 16;
+  const uint32_t S = w.S;
+  u32x4 x[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    uint32_t j = lane + v * kWave;
+    if (!EXACT) j = j < nvec ? j : nvec - 1;
+    x[v] = row[j];
+  }
+  float sc = 0.f;
+  const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
+  if (S) sc = sin[lane < S ? lane : S - 1];
+  // (pins the row loads in front of the branch below)
+#pragma unroll
+  for (int v = 0; v < NV; ++v) settle(x[v]);
+  settle(sc);
+  if (e >= w.E || slot == kInvalidSlot) return;
+  const DispatchRank &dst = tab.at(e / w.L);
+  const uint32_t el = e % w.L;
+  if (slot >= dst.x_rows) {
+    if (lane == 0) atomicOr(w.faults, kFaultRowDropped);
+    return;
+  }
+  PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
+      dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
+  PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
+                            (int64_t)slot * dst.xs_stride_row;
+  // same policy as the one-call dispatch: rows that fit the last-level cache stay there
+  if (write_through) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const uint32_t j = lane + v * kWave;
+      if (EXACT || j < nvec) row_store<RowStore::kKeep>(x[v], out + j);
+    }
+  } else {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const uint32_t j = lane + v * kWave;
+      if (EXACT || j < nvec) row_store<RowStore::kStreamThrough>(x[v], out + j);
+    }
+  }
+  if (lane < S) row_store<RowStore::kKeep>(sc, sout + (int64_t)lane * dst.xs_stride_elem);
+  for (uint32_t j = lane + kWave; j < S; j += kWave) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
+}
+
+// Rows beyond the register variants: one workgroup per (token, pick).
 template <class DT>
 __global__ __launch_bounds__(256) void split_unpack_long(WorldDev w, DT tab, SplitDev sp) {
-  const uint32_t e = blockIdx.x;
-  const uint32_t el = e % w.L;
+  publish_counts(w, tab, sp);
+  const uint64_t pair = blockIdx.x;
+  const uint32_t e = as_global(sp.gexp)[pair];
+  const uint32_t slot = as_global(w.slot_map)[pair];
+  if (e >= w.E || slot == kInvalidSlot) return;
   const DispatchRank &dst = tab.at(e / w.L);
-  const uint32_t count = as_global(sp.gcnt)[e], offset = as_global(sp.goff)[e];
-  if (blockIdx.y == 0 && threadIdx.x == 0) {
-    as_global(dst.out_num_tokens)[(int64_t)el * dst.out_num_tokens_stride] = (int32_t)count;
+  const uint32_t el = e % w.L;
+  if (slot >= dst.x_rows) {
+    if (threadIdx.x == 0) atomicOr(w.faults, kFaultRowDropped);
+    return;
   }
   const uint32_t nvec = w.Hb / 16;
-  for (uint32_t slot = blockIdx.y; slot < count; slot += gridDim.y) {
-    if (slot >= dst.x_rows) {
-      if (threadIdx.x == 0) atomicOr(w.faults, kFaultRowDropped);
-      continue;
-    }
-    const uint8_t *src = stage_row(sp, (uint64_t)offset + slot);
-    const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
-    PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
-        dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
-    for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
-    const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
-    PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
-                              (int64_t)slot * dst.xs_stride_row;
-    for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
-  }
+  const uint8_t *src = stage_row(sp, pair);
+  const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
+  PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(
+      dst.expert_x + (int64_t)el * dst.x_stride_expert + (int64_t)slot * dst.x_stride_row));
+  for (uint32_t j = threadIdx.x; j < nvec; j += blockDim.x) out[j] = row[j];
+  const PPLX_GLOBAL float *sin = as_global(reinterpret_cast<const float *>(src + w.Hb));
+  PPLX_GLOBAL float *sout = as_global(dst.expert_xs) + (int64_t)el * dst.xs_stride_expert +
+                            (int64_t)slot * dst.xs_stride_row;
+  for (uint32_t j = threadIdx.x; j < w.S; j += blockDim.x) sout[(int64_t)j * dst.xs_stride_elem] = sin[j];
 }
 
 // combine SEND: one wave per (token, pick) copies the expert_y row of the pick's expert into
@@ -237,28 +251,17 @@ __global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, Sp
 }
 
 template <class DT>
-int launch_split_dispatch_send_t(const WorldDev &w, const SplitDev &sp, const DT &tab, uint32_t pick_vector,
-                                 hipStream_t s) {
-  RouteSpan span{};
-  span.v_begin = 0;
-  span.v_count = w.G * w.M;
-  span.tile_chunks = w.tile_chunks;
-  span.pick_vector = pick_vector;
-  span.tile_cnt = w.tile_cnt;
-  span.slot_out = w.slot_map;
-  span.expert_out = sp.gexp;
-  span.counts_out = sp.gcnt;
-  span.offsets_out = sp.goff;
-  int err = launch_route_t<DT, true>(w, tab, span, s);
-  if (err) return err;
+int launch_split_pack_t(const WorldDev &w, const SplitDev &sp, const DT &tab, hipStream_t s) {
   const uint32_t lds = 0;
   const uint32_t tokens = w.G * w.M;
   if (!row_has_register_variant(w)) {
     hipLaunchKernelGGL(split_pack_long<DT>, dim3(tokens), dim3(256), 0, s, w, tab, sp);
     return (int)hipGetLastError();
   }
+  const uint64_t row_bytes = (uint64_t)tokens * w.K * sp.token_stride;
+  const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
   const dim3 grid((tokens + 3) / 4), block(256);
-#define PPLX_ROW_KERNEL_ARGS sp
+#define PPLX_ROW_KERNEL_ARGS sp, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(split_pack);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -269,21 +272,18 @@ int launch_split_dispatch_send_t(const WorldDev &w, const SplitDev &sp, const DT
 template <class DT>
 int launch_split_dispatch_recv_t(const WorldDev &w, const SplitDev &sp, const DT &tab, hipStream_t s) {
   const uint32_t lds = 0;
-  // Row groups per expert: enough workgroups to cover the CUs even with few experts, and a hot
-  // expert's long run is shared; never more than a run can use.
-  uint32_t spread = (2048 + w.E - 1) / w.E;
-  const uint64_t most = ((uint64_t)w.G * w.M + 3) / 4;
-  if (spread > most) spread = (uint32_t)most;
-  if (spread > 256) spread = 256;
-  if (spread < 1) spread = 1;
-  const dim3 grid(w.E, spread), block(256);
+  const uint64_t pairs = (uint64_t)w.G * w.M * w.K;
   if (!row_has_register_variant(w)) {
-    hipLaunchKernelGGL(split_unpack_long<DT>, grid, block, 0, s, w, tab, sp);
+    hipLaunchKernelGGL(split_unpack_long<DT>, dim3((uint32_t)pairs), dim3(256), 0, s, w, tab, sp);
     return (int)hipGetLastError();
   }
-  const uint64_t row_bytes = (uint64_t)w.G * w.M * w.K * (w.Hb + 4ull * w.S);
+  const uint64_t row_bytes = pairs * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
-#define PPLX_ROW_KERNEL_ARGS sp, write_through
+  // Small steps are mostly full (decode batches); the reads of empty pairs of a large ragged
+  // one would cost more than the trip saved.
+  const uint32_t eager = (uint64_t)w.G * w.M <= kFusedMaxTokens ? 1u : 0u;
+  const dim3 grid((uint32_t)((pairs + 3) / 4)), block(256);
+#define PPLX_ROW_KERNEL_ARGS sp, write_through, eager
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(split_unpack);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -303,12 +303,9 @@ int launch_split_combine_send_t(const WorldDev &w, const SplitDev &sp, const CT 
 
 }  // namespace
 
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
-                               uint32_t pick_vector, void *stream) {
-  if (pick_vector != 4 && pick_vector != 2) pick_vector = 1;
-  if (inline_rows)
-    return launch_split_dispatch_send_t(w, sp, make_inline(w, inline_rows), pick_vector, (hipStream_t)stream);
-  return launch_split_dispatch_send_t(w, sp, HbmDispatch{w.drank}, pick_vector, (hipStream_t)stream);
+int launch_split_pack(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows, void *stream) {
+  if (inline_rows) return launch_split_pack_t(w, sp, make_inline(w, inline_rows), (hipStream_t)stream);
+  return launch_split_pack_t(w, sp, HbmDispatch{w.drank}, (hipStream_t)stream);
 }
 
 int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
