@@ -745,7 +745,7 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
   } allocs[] = {
       {reinterpret_cast<void **>(&d.drank), sizeof(DispatchRank) * d.R},
       {reinterpret_cast<void **>(&d.crank), sizeof(CombineRank) * d.R},
-      {reinterpret_cast<void **>(&d.tile_cnt), sizeof(uint32_t) * (size_t)d.num_tiles * d.E},
+      {reinterpret_cast<void **>(&d.tile_cnt), (size_t)route_tables(d.num_tiles, d.tile_chunks, d.E).bytes},
       {reinterpret_cast<void **>(&d.slot_map), sizeof(uint32_t) * (size_t)d.G * d.M * d.K},
       {reinterpret_cast<void **>(&d.faults), 256},
   };
@@ -959,9 +959,9 @@ int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
   WorldDev d{};
   fill_geometry(*cfg, d);
   // Scratch layout: the fault word, the slot map (the hand-off from dispatch to combine, kept
-  // from one call to the next), the routing tiles' counts.
+  // from one call to the next), the routing tiles' counts and masks.
   const size_t slot_bytes = sizeof(uint32_t) * (size_t)d.G * d.M * d.K;
-  const size_t tile_bytes = sizeof(uint32_t) * (size_t)d.num_tiles * d.E;
+  const size_t tile_bytes = (size_t)route_tables(d.num_tiles, d.tile_chunks, d.E).bytes;
   const size_t slot_at = 256, tile_at = slot_at + (slot_bytes + 255) / 256 * 256;
   const size_t needed = tile_at + tile_bytes;
   if (needed > kStaticScratchBytes)

@@ -77,10 +77,25 @@ struct WorldDev {
   DispatchRank *drank;   // [R]
   CombineRank *crank;    // [R]
   uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile; after route_scan the
-                         // tokens routed to e in all earlier tiles
+                         // tokens routed to e in all earlier tiles.  Behind it (route_tables):
+                         // [num_tiles * tile_chunks][E] 64-bit masks, one bit per token of a chunk
   uint32_t *slot_map;    // [G * M][K] row of (token, pick) inside its expert
   uint32_t *faults;      // [1] sticky fault bits
 };
+
+// The routing scratch of a world is one block: the tiles' counts, then the chunks' masks.
+struct RouteTables {
+  uint64_t mask_offset, bytes;
+};
+#ifdef __HIPCC__
+__host__ __device__
+#endif
+inline RouteTables route_tables(uint32_t num_tiles, uint32_t tile_chunks, uint32_t experts) {
+  RouteTables t;
+  t.mask_offset = ((uint64_t)num_tiles * experts * 4u + 7u) & ~7ull;
+  t.bytes = t.mask_offset + (uint64_t)num_tiles * tile_chunks * experts * 8u;
+  return t;
+}
 
 // Which virtual tokens a routing launch covers and where its results go.
 struct RouteSpan {
@@ -89,6 +104,9 @@ struct RouteSpan {
   uint32_t tile_chunks;   // 64-token chunks per tile (one workgroup)
   uint32_t pick_vector;   // expert ids one load may fetch (4, 2 or 1)
   uint32_t *tile_cnt;     // [tiles][E]
+  unsigned long long *tile_mask;  // [tiles * tile_chunks][E] route_count keeps the chunks' masks
+                                  // here (and reports the faults) when set: the scatter that
+                                  // follows works the slots out by itself
   uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
   // split mode only:
   uint32_t *expert_out;   // [G * M][K] expert of every pair (num_experts = the pair has no row)

@@ -44,10 +44,11 @@ __global__ __launch_bounds__(256) void bind_rows(Row *table, Batch b) {
   }
 }
 
-// Launched as one-wave workgroups whose dynamic LDS size caps how many of them a CU holds at a
-// time (see launch_scatter_t); the kernel itself does not touch LDS.
-template <int NV, bool EXACT, class DT>
-__global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+// One wave per token (or per share of its picks).  ROUTED: the slot map was written by
+// route_slots; otherwise the wave works its token's slots out of the routing tables
+// (slots_from_masks) and writes the slot map itself.
+template <int NV, bool EXACT, class DT, bool ROUTED>
+__device__ __forceinline__ void scatter_token(const WorldDev &w, const DT &tab, uint32_t ksplit, uint32_t kper) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
                                                        threadIdx.x / kWave);
@@ -62,10 +63,19 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   RowRegs<NV> regs;
   load_row<NV, EXACT>(w, src, t, lane, regs);
   Destination dst;
-  if (lane < w.K) {
-    dst = resolve_destination(w, tab, as_global(src.indices)[(size_t)t * w.K + lane],
-                              as_global(w.slot_map)[(size_t)v * w.K + lane],
-                              part == 0);
+  if constexpr (ROUTED) {
+    if (lane < w.K) {
+      dst = resolve_destination(w, tab, as_global(src.indices)[(size_t)t * w.K + lane],
+                                as_global(w.slot_map)[(size_t)v * w.K + lane],
+                                part == 0);
+    }
+  } else {
+    const uint32_t e = lane < w.K ? as_global(src.indices)[(size_t)t * w.K + lane] : w.E;
+    const uint32_t slot = slots_from_masks(w, v, lane, e);
+    if (lane < w.K) {
+      dst = resolve_destination(w, tab, e, slot, part == 0);
+      if (part == 0) as_global(w.slot_map)[(size_t)v * w.K + lane] = slot;
+    }
   }
   const uint32_t k0 = part * kper;
   const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
@@ -73,6 +83,18 @@ __global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint
   // last-level cache instead, where the partial lines of neighbouring rows meet before they go
   // to HBM (3-4 % of the kernel's time at 224-byte scale rows).
   store_row<NV, EXACT, RowStore::kStreamThrough, RowStore::kKeep>(w, src, t, lane, dst, k0, k1, regs);
+}
+
+// Launched as one-wave workgroups whose dynamic LDS size caps how many of them a CU holds at a
+// time (see launch_scatter_t); the kernels themselves do not touch LDS.
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void dispatch_scatter(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+  scatter_token<NV, EXACT, DT, true>(w, tab, ksplit, kper);
+}
+
+template <int NV, bool EXACT, class DT>
+__global__ __launch_bounds__(256) void dispatch_scatter_slots(WorldDev w, DT tab, uint32_t ksplit, uint32_t kper) {
+  scatter_token<NV, EXACT, DT, false>(w, tab, ksplit, kper);
 }
 
 // Threads of a dispatch_fused workgroup: 16 waves (fewer, larger workgroups repeat less
@@ -433,31 +455,36 @@ uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
 }
 
 // Scatter waves a CU should hold at a time (0 = as many as fit).
-// Measured on 8 x 4096 tokens (us at 2 / 3 / 4 / 6 / 8 waves per CU / full occupancy):
-//   59 KiB stored per wave (DSv3 fp8 rows, top-8)     419 / 423 / 439 / 444 / 441 / 449
-//   32 KiB (4 KiB rows, top-8)                        210 / 213 / 217 / 220 / 221 / 227
-//   16 KiB (8 KiB rows, top-2)                        180 / 153 / 153 / 163 / 165 / 170
-//   17 KiB (2 KiB fp8 rows with scales, top-8)        178 / 137 / 119 / 110 / 111 / 117
-//    8 KiB (1 KiB rows, top-8)                        128 /  95 /  80 /  65 /  59 /  65
-//    4 KiB (2 KiB rows, top-2)                        112 /  85 /  72 /  59 /  53 /  46
-// and on the large prefill with ragged token counts and skewed routing (8 x <= 8192 DSv3 tokens):
-// 457 / 447 / 459 us at 2 / 3 / 4, 474 us at full occupancy.  A wave's loads and launch are
-// dead time for the stores, so the less a wave stores the more of them it takes to keep the
-// CU's stores going.
+// Measured on 8 x 4096 tokens with the slots worked out by the scatter's waves
+// (us at 3 / 4 / 6 / 8 / 12 / 16 waves per CU / full occupancy):
+//   112 KiB stored per wave (14 KiB rows, top-8)      847 / 844 / 851 / 855 / 860 / 858 / 857
+//   59 KiB (DSv3 fp8 rows, top-8)                     404 / 421 / 437 / 437 / 427 / 432 / 433
+//   32 KiB (4 KiB rows, top-8)                        206 / 211 / 215 / 216 / 217 / 220 / 221
+//   16 KiB (8 KiB rows, top-2)                        164 / 152 / 155 / 160 / 163 / 165 / 167
+//   17 KiB (2 KiB fp8 rows with scales, top-8)        163 / 133 / 106 / 104 / 109 / 110 / 111
+//   14 KiB (DSv3 fp8 rows, top-2)                     181 / 155 / 140 / 141 / 146 / 149 / 148
+//    8 KiB (1 KiB rows, top-8)                        122 / 100 /  77 /  64 /  57 /  60 /  60
+//    4 KiB (2 KiB rows, top-2)                        103 /  84 /  66 /  57 /  50 /  46 /  44
+// and on the Mixtral prefill (8 x 4096 tokens of 8 KiB, top-2, skewed routing) 147.5 us at 4
+// against 145.8 at 6.  A wave's launch, its loads and its slot arithmetic are dead time for the
+// stores, so the less a wave stores the more of them it takes to keep the CU's stores going.
 uint32_t scatter_waves_per_cu(const WorldDev &w, uint32_t picks_per_wave) {
   if (w.lds_per_cu == 0) return 0;
   const uint64_t row = w.Hb + 4ull * w.S;
   const uint64_t stored = (uint64_t)picks_per_wave * row;
   if (stored >= 24 * 1024) return 3;
-  if (stored >= 12 * 1024) return row >= 4096 ? 4 : 6;
-  if (stored >= 6 * 1024) return 8;
+  if (stored >= 12 * 1024) return row >= 4096 ? 6 : 8;
+  if (stored >= 6 * 1024) return 12;
   return 0;
 }
 
+// Rows that dispatch_scatter holds in registers (longer ones stream through dispatch_scatter_long).
+bool scatter_has_register_rows(const WorldDev &w) { return (w.Hb / 16 + kWave - 1) / kWave <= 32; }
+
 template <class DT>
-int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
+int launch_scatter_t(const WorldDev &w, const DT &tab, bool routed, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
-  if ((w.Hb / 16 + kWave - 1) / kWave > 32) {
+  if (!scatter_has_register_rows(w)) {
     hipLaunchKernelGGL(dispatch_scatter_long<DT>, dim3(tokens), dim3(256), 0, s, w, tab);
     return (int)hipGetLastError();
   }
@@ -481,7 +508,11 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, hipStream_t s) {
     if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                              \
     else PPLX_LAUNCH_ROW_VARIANT(KERNEL, 32, false);                                             \
   } while (0)
-  PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
+  if (routed) {
+    PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
+  } else {
+    PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter_slots);
+  }
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
 #undef PPLX_ROW_KERNEL_ARGS
   return (int)hipGetLastError();
@@ -526,9 +557,16 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hi
   span.pick_vector = pick_vector;
   span.tile_cnt = w.tile_cnt;
   span.slot_out = w.slot_map;
+  // Steps of several tiles leave the last routing launch out: the scatter's waves work their
+  // own slots out of the tiles' tables.
+  const bool slots_in_scatter = w.num_tiles > 1 && scatter_has_register_rows(w);
+  if (slots_in_scatter) {
+    span.tile_mask = reinterpret_cast<unsigned long long *>(
+        reinterpret_cast<uint8_t *>(w.tile_cnt) + route_tables(w.num_tiles, w.tile_chunks, w.E).mask_offset);
+  }
   int err = launch_route_t<DT, false>(w, tab, span, s);
   if (err) return err;
-  return launch_scatter_t(w, tab, s);
+  return launch_scatter_t(w, tab, !slots_in_scatter, s);
 }
 
 }  // namespace

@@ -19,6 +19,9 @@ namespace {
 //   route_slots   per tile: the masks again, slots               -> slot map
 // An expert id repeated inside one token sets its bit once: the repeat takes no row, is not
 // counted, and is reported (kFaultDuplicateExpert).
+// With span.tile_mask set, route_count also keeps the masks and reports the faults, and there
+// is no route_slots launch: the scatter that follows works each token's slots out of the
+// scanned counts and the masks by itself (slots_from_masks).
 //
 // SPLIT = false: the launch writes out_expert_num_tokens of the owning ranks.  SPLIT = true
 // (dispatch SEND of split mode, which may not touch the outputs yet): the rows per expert go to
@@ -63,12 +66,15 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpa
   const RouteToken tok = route_token(w, tab, span);
   // (the picks are fetched whenever their row exists, behind the group's token count and not
   // after it: one trip to memory instead of two)
+  uint32_t codes = 0;
   if (tok.row_exists) {
     const bool live = tok.t < tok.n_group;
-    for_each_pick<PV>(tok.idx, w.K, [&](uint32_t, uint32_t e) __attribute__((always_inline)) {
-      if (live && e < w.E) atomicOr(&lds_mask[(size_t)chunk * w.E + e], 1ull << lane);
-      return 0u;
-    });
+    codes = for_each_pick<PV>(tok.idx, w.K, [&](uint32_t, uint32_t e) __attribute__((always_inline)) {
+      if (!live) return 0u;
+      if (e >= w.E) return kFaultBadExpert;
+      const unsigned long long bit = 1ull << lane;
+      return (atomicOr(&lds_mask[(size_t)chunk * w.E + e], bit) & bit) ? kFaultDuplicateExpert : 0u;
+    }).codes;
   }
   __syncthreads();
   uint32_t *out = span.tile_cnt + (size_t)blockIdx.x * w.E;
@@ -77,6 +83,49 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpa
     for (uint32_t c = 0; c < chunks; ++c) rows += __popcll(lds_mask[(size_t)c * w.E + e]);
     out[e] = rows;
   }
+  if (span.tile_mask != nullptr) {
+    unsigned long long *keep = span.tile_mask + (size_t)blockIdx.x * chunks * w.E;
+    for (uint32_t i = threadIdx.x; i < chunks * w.E; i += blockDim.x) keep[i] = lds_mask[i];
+    if (codes) atomicOr(w.faults, codes);
+    if (tok.in_span && tok.t == 0 && dispatch_group_overflows(w, tab, tok.g)) {
+      atomicOr(w.faults, kFaultTooManyTokens);
+    }
+  }
+}
+
+// What route_slots would have written for pick `lane` of virtual token v (wave-uniform), from
+// the scanned counts and the masks that route_count kept: rows of earlier tiles + rows of
+// earlier chunks of the tile + earlier tokens of the chunk.  A pick that repeats an earlier
+// one of its token, or names no expert, has no row.
+__device__ __forceinline__ uint32_t slots_from_masks(const WorldDev &w, uint32_t v, uint32_t lane, uint32_t e) {
+  const uint32_t chunks = w.tile_chunks;
+  const uint32_t chunk_abs = v / kWave;
+  const uint32_t tile = chunk_abs / chunks;
+  const uint32_t c = chunk_abs - tile * chunks;
+  const unsigned long long below = (1ull << (v & (kWave - 1))) - 1ull;
+  bool has_row = lane < w.K && e < w.E;
+  for (uint32_t k = 0; k + 1 < w.K; ++k) {
+    const uint32_t earlier = (uint32_t)__builtin_amdgcn_readlane((int)e, (int)k);
+    if (lane > k && earlier == e) has_row = false;
+  }
+  if (!has_row) return kInvalidSlot;
+  const PPLX_GLOBAL unsigned long long *mask =
+      as_global(reinterpret_cast<const unsigned long long *>(
+          reinterpret_cast<const uint8_t *>(w.tile_cnt) + route_tables(w.num_tiles, chunks, w.E).mask_offset)) +
+      (size_t)tile * chunks * w.E + e;
+  uint32_t slot = as_global(w.tile_cnt)[(size_t)tile * w.E + e];
+  // four masks per trip (tiles of four chunks: one trip)
+  for (uint32_t c0 = 0; c0 <= c; c0 += 4) {
+    unsigned long long m[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) m[i] = mask[(size_t)(c0 + i <= c ? c0 + i : c) * w.E];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      if (c0 + i < c) slot += __popcll(m[i]);
+      if (c0 + i == c) slot += __popcll(m[i] & below);
+    }
+  }
+  return slot;
 }
 
 // One wavefront per expert: tile_cnt[.][e] becomes its own exclusive prefix over the tiles, and
@@ -205,6 +254,7 @@ int launch_route_pv(const WorldDev &w, const DT &tab, const RouteSpan &span, hip
     hipLaunchKernelGGL((route_scan<DT, SPLIT>), dim3((w.E + 3) / 4), dim3(256), 0, s, w, tab, span, tiles);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return (int)err;
+    if (span.tile_mask != nullptr) return 0;  // the scatter works the slots out
   }
   hipLaunchKernelGGL((route_slots<DT, SPLIT, PV>), dim3(tiles), dim3(block), lds, s, w, tab, span,
                      tiles > 1 ? 1u : 0u);

@@ -72,7 +72,8 @@ def _combine_kw(step, r):
 def _check_with_repeats_dropped(step, after_combine: bool):
     """Literal expectation for a step whose tokens may repeat an expert: walking groups, tokens
     and picks in order, a pick takes the next row of its expert unless the token already named
-    that expert (tests/test_all_to_all.py:113-120 appends a token to an expert's list once)."""
+    that expert (tests/test_all_to_all.py:113-120 appends a token to an expert's list once).  A
+    pick that names no expert takes no row either, and rows beyond the capacity are not there."""
     spec, groups = step.spec, step.groups
     E, K, H = spec.num_experts, spec.experts_per_token, spec.hidden_dim
     rows_of = [[] for _ in range(E)]
@@ -82,7 +83,7 @@ def _check_with_repeats_dropped(step, after_combine: bool):
             seen = set()
             for k in range(K):
                 e = int(grp.indices[t, k])
-                if e in seen:
+                if e in seen or e >= E:
                     slot_of[(g, t, k)] = None
                     continue
                 seen.add(e)
@@ -94,7 +95,7 @@ def _check_with_repeats_dropped(step, after_combine: bool):
     got_x = step.expert_x_all.view(torch.uint8).reshape(E, step.cap, -1).cpu().numpy()
     got_s = step.expert_x_scale_all.reshape(E, step.cap, -1).cpu().numpy() if spec.scale_dim else None
     for e in range(E):
-        for s_, (g, t) in enumerate(rows_of[e]):
+        for s_, (g, t) in enumerate(rows_of[e][: step.cap]):
             want = groups[g].x[t].contiguous().view(torch.uint8).numpy()
             np.testing.assert_array_equal(got_x[e, s_], want)
             if got_s is not None:
@@ -123,6 +124,8 @@ def _check_with_repeats_dropped(step, after_combine: bool):
         dict(name="dup-top12", experts_per_token=12, num_experts=32),
         # more than 3072 virtual tokens: routing tiles + scatter
         dict(name="dup-tiles", max_num_tokens=4200, experts_per_token=2),
+        # tiles of eight chunks, groups that start in the middle of a tile
+        dict(name="dup-wide-tiles", max_num_tokens=20000, experts_per_token=8, num_experts=32, in_dtype=FP8, hidden_dim=512),
     ],
     ids=lambda kw: kw["name"],
 )
@@ -155,6 +158,29 @@ def test_repeated_expert_is_dropped_and_reported(kw):
     step.combine_world(world)
     assert world.faults() == 0
     _check_with_repeats_dropped(step, after_combine=True)
+    world.destroy()
+
+
+def test_faults_of_a_step_of_several_routing_tiles():
+    """A pick that names no expert and an expert with more rows than its buffer holds, in the
+    dispatch form whose scatter works the slots out itself: both are reported, the counts give
+    the full demand and every row that fits is in place."""
+    spec = _spec(name="tiles-faults", max_num_tokens=4200, experts_per_token=4)
+    groups = generate(spec)
+    for g in groups:
+        g.n = min(max(g.n, 8), 200)
+    groups[1].indices[3, 1] = 999
+    counts = np.zeros(spec.num_experts, dtype=np.int64)
+    for g in groups:
+        ids = g.indices[: g.n].numpy().reshape(-1)
+        counts += np.bincount(ids[ids < spec.num_experts], minlength=spec.num_experts)
+    step = DeviceStep(spec, groups, cap=int(counts.max()) - 2)
+    world = make_world(spec, group_name="tiles-faults")
+    step.dispatch_world(world)
+    torch.cuda.synchronize()
+    assert world.faults() == FAULT_ROW_DROPPED | FAULT_BAD_EXPERT
+    np.testing.assert_array_equal(step.expert_num_tokens_all.cpu().numpy().reshape(-1), counts)
+    _check_with_repeats_dropped(step, after_combine=False)
     world.destroy()
 
 
