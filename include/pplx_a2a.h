@@ -191,10 +191,11 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *world, const pplx_a2a_combine_args_
  * forbid hipMalloc.  `dispatch_per_rank` / `combine_per_rank` are host arrays
  * of world_size entries as for pplx_a2a_world_dispatch / _combine (either may be
  * NULL to skip that half); the kernels and the results are the same.  The state
- * a world would own (slot map, routing tile counts) lives in a 4 MiB array that
+ * a world would own (slot map, routing tables) lives in an 8 MiB array that
  * is part of the library's code object on every GPU; a geometry that needs more
  * (world_size / dp_size * max_num_tokens * experts_per_token * 4 bytes of slot
- * map plus the tile counts), or more than 64 ranks, is refused with
+ * map plus about world_size / dp_size * max_num_tokens * num_experts / 8 bytes of
+ * routing tables), or more than 64 ranks, is refused with
  * PPLX_A2A_INVALID_ARGUMENT / PPLX_A2A_UNSUPPORTED.  The slot map written by a
  * dispatch stays there for the combine of a later call.  All calls on one GPU
  * share the array: calls that overlap in time on one GPU (different streams or

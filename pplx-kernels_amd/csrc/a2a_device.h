@@ -164,7 +164,7 @@ constexpr uint64_t kWriteThroughMaxBytes = 128ull << 20;
 
 // Device memory that pplx_a2a_static_step works in instead of a world's allocations: a fixed
 // array inside the library's code object (a2a_static.hip), one copy per GPU.
-constexpr size_t kStaticScratchBytes = 4u << 20;
+constexpr size_t kStaticScratchBytes = 8u << 20;
 // Address of the calling thread's current device's copy (looked up once per device).
 int static_scratch_address(int device, void **out);
 
