@@ -468,3 +468,16 @@ def test_cpp_benchmark_runs_the_reference_sequence():
     assert "send+recv against one call" in proc.stdout
     assert "overlap," in proc.stdout
     assert np.isfinite(float(proc.stdout.split("send+recv against one call: dispatch ")[1].split("x")[0]))
+
+
+def test_cpp_memory_yardstick_runs():
+    """The plain streaming kernels that the achieved rates are read against: every line reports
+    a rate below the published peak and above a tenth of it."""
+    exe = os.path.join(ROOT, "pplx-kernels_amd", "bin", "bench_hbm")
+    assert os.path.exists(exe), "build it with `make -C pplx-kernels_amd/csrc`"
+    proc = subprocess.run([exe, "3"], capture_output=True, text=True, timeout=300)
+    print(proc.stdout[-3000:], proc.stderr[-2000:])
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    rates = [float(line.split("TB/s")[0].split()[-1]) for line in proc.stdout.splitlines() if "TB/s " in line]
+    assert len(rates) == 15
+    assert all(0.8 < r < 8.0 for r in rates), rates
