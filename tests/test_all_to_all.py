@@ -499,6 +499,16 @@ def test_more_ranks_than_inline_tables_hold(api):
     run_and_check(spec, generate(spec), api=api)
 
 
+def test_more_ranks_than_inline_tables_hold_in_a_step_of_several_tiles():
+    """72 ranks x 50 tokens: the HBM-table variants of the routing kernels and of the scatter
+    that works its slots out."""
+    spec = _small_spec(
+        name="r72-tiles", world_size=72, num_experts=144, experts_per_token=4, max_num_tokens=50,
+        hidden_dim=512, in_dtype=FP8,
+    )  # fmt: skip
+    run_and_check(spec, generate(spec), api="world")
+
+
 def test_hbm_tables_under_graph_replay():
     """A captured step of a > 64-rank world re-binds its tables on every replay, also after
     eager calls with other tensors have rewritten them."""
