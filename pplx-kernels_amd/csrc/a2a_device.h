@@ -160,7 +160,7 @@ constexpr uint32_t kBindBatch = 64;
 constexpr uint32_t kFusedMaxTokens = 3072;
 // A fused launch whose rows (all picks of all tokens) stay within this many bytes stores them
 // write-through into the 256 MB last-level cache instead of streaming them past it.
-constexpr uint64_t kWriteThroughMaxBytes = 128ull << 20;
+constexpr uint64_t kWriteThroughMaxBytes = 192ull << 20;
 
 // Device memory that pplx_a2a_static_step works in instead of a world's allocations: a fixed
 // array inside the library's code object (a2a_static.hip), one copy per GPU.

@@ -7,11 +7,14 @@
 // placement is the canonical (expert, DP group, token) order that the
 // reference's tests enumerate (tests/test_all_to_all.py:113-120):
 //
-//   route_count      per routing tile: histogram of expert ids        (only if > 1 tile)
-//   route_slots      per routing tile: 64-token bitmasks per expert in LDS,
-//                    prefix over chunks and earlier tiles -> slot_map, counts
-//   dispatch_scatter one wave per token (or per share of its K picks): the row
-//                    is read once into registers and stored K times, 16 B / lane
+//   route_count      per routing tile: 64-token bitmasks per expert in LDS -> rows per
+//                    expert of the tile, and the masks themselves          (only if > 1 tile)
+//   route_scan       per expert: prefix of the tiles' rows, totals         (only if > 1 tile)
+//   dispatch_scatter_slots  one wave per token (or per share of its K picks): the row is
+//                    read once into registers, lane k works the slot of pick k out of the
+//                    scanned rows and the masks, the row is stored K times, 16 B / lane
+//   route_slots + dispatch_scatter  the same with the slots written by a launch of their
+//                    own (single tile, rows beyond the register variants)
 //   dispatch_fused   small steps: routing and scatter in one launch; every
 //                    workgroup recounts the picks of the tokens before its own
 //   combine_gather   one wave per 1 KiB of an output row: K rows gathered through
@@ -580,11 +583,12 @@ uint32_t route_lds_bytes(uint32_t num_experts, uint32_t tile_chunks) {
 
 bool dispatch_is_fused(const WorldDev &w) {
   // Every workgroup recounts all earlier tokens (work that grows with the square of the token
-  // count) and all sixteen waves of a workgroup store at once, while the scatter of the
-  // three-to-four-launch form keeps few storing waves per CU.  Measured at 7 KiB rows, top-8, 8
-  // ranks (one launch / routing + scatter): 2048 tokens 24 / 42 us, 4096 tokens 61.5 / 58.8 us,
-  // 8192 tokens 109 / 100 us: the one-launch form pays while the routing launches (about 16 us of
-  // latency) weigh more than the scatter's better rate.
+  // count) and all of a workgroup's row waves store at once, while the scatter behind the two
+  // routing launches keeps few storing waves per CU.  Measured on 8 ranks (us, one launch /
+  // routing + scatter) at 2048, 3072, 4096, 6144 tokens: 7 KiB fp8 rows, top-8 of 256:
+  // 24 / 37, 45 / 48, 61 / 56, 86 / 79; 8 KiB rows, top-2 of 8: 15 / 21, 20 / 25, 26 / 27,
+  // 40 / 35; 4 KiB rows, top-8 of 64: 19 / 25, 26 / 32, 34 / 36, 49 / 49.  The one-launch form pays
+  // while the routing launches (about 10 us of latency) weigh more than the scatter's better rate.
   const uint64_t tokens = (uint64_t)w.G * w.M;
   return tokens <= kFusedMaxTokens && row_has_register_variant(w) && fused_lds_bytes(w, 16, true) <= 60 * 1024;
 }
