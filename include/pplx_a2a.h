@@ -131,7 +131,10 @@ typedef struct pplx_a2a_combine_args {
 
 /* ---- lifecycle ------------------------------------------------------- */
 
-/* Allocates the world's device state on `device` (a HIP device ordinal).
+/* Allocates the world's device state on `device` (a HIP device ordinal): with
+ * T = world_size / dp_size * max_num_tokens, a slot map of T * experts_per_token * 4
+ * bytes and routing tables of about T * num_experts / 8 bytes (the 8192-token
+ * DSv3 shape: 2 MiB + 2.3 MiB), plus rank tables for worlds of more than 64 ranks.
  * Replaces the buffer set-up of csrc/all_to_all/intranode.cpp:11-137. */
 int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_world_t **out);
 /* Frees the world.  Fails with INVALID_STATE while rank handles are attached. */
