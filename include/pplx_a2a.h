@@ -205,11 +205,36 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *world, const pplx_a2a_combine_args_
  * threads) race, and a step of a different geometry overwrites the slot map.
  * `fault_bits`: optional device word that the kernels OR the fault bits of
  * pplx_a2a_world_faults into (the caller clears and reads it); NULL discards them.
- * Calls no hipMalloc / hipFree and never synchronises. */
+ * Calls no hipMalloc / hipFree and never synchronises.  The first call on a device looks the
+ * array's address up (pplx_a2a_world_create on that device does the same): it cannot be made
+ * under stream capture and returns PPLX_A2A_INVALID_STATE there. */
 int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
                          const pplx_a2a_dispatch_args_t *dispatch_per_rank,
                          const pplx_a2a_combine_args_t *combine_per_rank, uint32_t *fault_bits,
                          void *stream);
+
+/* Parts of a step for pplx_a2a_world_abandon_step. */
+#define PPLX_A2A_ABANDON_DISPATCH 1u
+#define PPLX_A2A_ABANDON_COMBINE 2u
+
+/* Drops the calls recorded so far for the dispatch and / or combine step (or split phase)
+ * that is being assembled and returns that half of the world to idle, so that every rank can
+ * call again.  For the caller whose rank r fails its argument checks after other ranks of the
+ * step have called: nothing of a step reaches the GPU before its last rank has called, so the
+ * recorded calls are forgotten and no kernel runs.  A split step between its SEND and RECV
+ * phases is given up as a whole (what SEND staged is overwritten by the next SEND).
+ * `dropped_calls` (optional) receives the number of recorded calls that were dropped.  The
+ * reference has no such exit because it has no such state: a failed check there ends the
+ * process (csrc/core/cuda_utils.h:7-14, csrc/core/utils.h:16-24).  Only host state changes:
+ * no allocation, no synchronisation. */
+int pplx_a2a_world_abandon_step(pplx_a2a_world_t *world, uint32_t which, uint32_t *dropped_calls);
+/* Number of per-rank calls of `op` (0 = dispatch, 1 = combine) in `split_mode` that the world
+ * has recorded and not launched yet; 0 once the last rank's call has enqueued the phase.  A
+ * binding that keeps the callers' buffers alive for the ranks that called early reads this to
+ * know when to let them go. */
+int pplx_a2a_world_recorded_calls(pplx_a2a_world_t *world, int op, int split_mode, uint32_t *out);
+/* The world a rank handle is attached to. */
+pplx_a2a_world_t *pplx_a2a_world_of(const pplx_a2a_t *handle);
 
 /* Allocates the staging that split send / recv calls go through (the reference
  * allocates its inboxes in the constructor, csrc/all_to_all/intranode.cpp:37-136;
@@ -217,7 +242,10 @@ int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
  * G*M*K * (hidden_dim_bytes + hidden_dim_scale_bytes + 16) bytes for dispatch plus
  * G*M*K * hidden_dim * expert_y_elem_bytes for combine (0 = dispatch only, 2 =
  * bf16 / f16 expert_y, 4 = also f32).  May be called again with a wider element
- * while no split combine step is in flight.  Synchronises the device. */
+ * while no split combine step is in flight, which frees the narrower combine staging: once a
+ * stream capture has recorded split calls of the world the graph holds that address, and a
+ * widening call returns PPLX_A2A_INVALID_STATE (reserve the widest element before capturing).
+ * Synchronises the device. */
 int pplx_a2a_world_reserve_split(pplx_a2a_world_t *world, uint32_t expert_y_elem_bytes);
 
 /* Reads and clears the world's device-side fault word (synchronises `stream`):

@@ -135,6 +135,9 @@ struct pplx_a2a_world {
   std::vector<uint8_t> dsend, drecv, csend, crecv;
   uint32_t n_dsend = 0, n_drecv = 0, n_csend = 0, n_crecv = 0;
   int split_in_dtype = -1;
+  // A stream capture has recorded split-mode kernels: the graph holds the staging addresses as
+  // kernel arguments, so the staging may no longer move.
+  bool split_captured = false;
 };
 
 struct pplx_a2a {
@@ -518,6 +521,13 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
   if (y_elem_bytes > w.split_y_elem_bytes) {
     if (w.n_csend != 0 || w.n_crecv != 0)
       return fail(PPLX_A2A_INVALID_STATE, "a split combine step is in flight");
+    // Widening frees the old combine staging.  A graph that recorded split calls carries its
+    // address and would write through it on the next replay.
+    if (w.split_captured && w.split.stage_y != nullptr)
+      return fail(PPLX_A2A_INVALID_STATE,
+                  "split calls of this world have been captured into a graph, which holds the address of the "
+                  "combine staging: it cannot be widened to %u-byte elements any more (reserve the widest "
+                  "expert_y element before capturing)", y_elem_bytes);
     // stage_y holds one expert_y row per (token, pick)
     HIP_TRY(hipDeviceSynchronize());
     (void)hipFree(sp.stage_y);
@@ -552,6 +562,7 @@ int run_split_dispatch(pplx_a2a_world &w, int mode, void *stream) {
   int st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
+  if (session != 0) w.split_captured = true;
   const DispatchRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_dispatch.data() : nullptr;
   if (!inline_rows) {
     st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
@@ -614,6 +625,7 @@ int run_split_combine(pplx_a2a_world &w, int mode, int in_dtype, int out_dtype, 
   int st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_combine, w.bound_combine_valid);
+  if (session != 0) w.split_captured = true;
   const CombineRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_combine.data() : nullptr;
   if (!inline_rows) {
     st = flush_table<CombineRank, BindCombineBatch>(w, w.pend_combine, w.bound_combine, w.bound_combine_valid,
@@ -696,7 +708,7 @@ extern "C" {
 
 const char *pplx_a2a_last_error(void) { return g_last_error.c_str(); }
 
-const char *pplx_a2a_version(void) { return "0.2.0"; }
+const char *pplx_a2a_version(void) { return "0.3.0"; }
 
 #ifndef PPLX_A2A_SOURCE_ID
 #define PPLX_A2A_SOURCE_ID "unknown"
@@ -718,8 +730,9 @@ int pplx_a2a_world_create(const pplx_a2a_config_t *cfg, int device, pplx_a2a_wor
   {
     // The first world on a device also looks up that device's copy of the library's static
     // scratch array, so that pplx_a2a_static_step finds it ready.
+    // (a world does not need the array: a failed lookup is left for that entry point to report)
     void *unused = nullptr;
-    LAUNCH_TRY(static_scratch_address(device, &unused));
+    (void)static_scratch_address(device, &unused);
   }
   pplx_a2a_world *w = new (std::nothrow) pplx_a2a_world();
   if (!w) return fail(PPLX_A2A_HIP_ERROR, "out of host memory");
@@ -849,6 +862,8 @@ uint64_t pplx_a2a_num_experts_per_token(const pplx_a2a_t *h) { return h ? h->wor
 
 uint32_t pplx_a2a_rank(const pplx_a2a_t *h) { return h ? h->rank : 0; }
 
+pplx_a2a_world_t *pplx_a2a_world_of(const pplx_a2a_t *h) { return h ? h->world : nullptr; }
+
 int pplx_a2a_dispatch(pplx_a2a_t *h, const pplx_a2a_dispatch_args_t *args, int split_mode,
                       void *stream) {
   if (!h || !args) return fail(PPLX_A2A_INVALID_ARGUMENT, "handle / args is NULL");
@@ -938,6 +953,58 @@ int pplx_a2a_world_combine(pplx_a2a_world_t *w, const pplx_a2a_combine_args_t *p
   return run_combine(*w, stream);
 }
 
+int pplx_a2a_world_recorded_calls(pplx_a2a_world_t *w, int op, int split_mode, uint32_t *out) {
+  if (!w || !out) return fail(PPLX_A2A_INVALID_ARGUMENT, "world / out is NULL");
+  if ((op != 0 && op != 1) || split_mode < PPLX_A2A_SPLIT_NONE || split_mode > PPLX_A2A_SPLIT_RECV)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "op must be 0 (dispatch) or 1 (combine), split_mode a pplx_a2a_split_mode");
+  std::lock_guard<std::mutex> lock(w->mu);
+  const uint32_t R = w->dev.R;
+  // (a phase whose count has reached world_size has been launched: nothing of it is pending)
+  auto pending = [R](uint32_t count) { return count < R ? count : 0u; };
+  if (split_mode == PPLX_A2A_SPLIT_NONE) {
+    *out = op == 0 ? w->n_arrived_dispatch : w->n_arrived_combine;
+  } else if (split_mode == PPLX_A2A_SPLIT_SEND) {
+    *out = pending(op == 0 ? w->n_dsend : w->n_csend);
+  } else {
+    *out = pending(op == 0 ? w->n_drecv : w->n_crecv);
+  }
+  return PPLX_A2A_OK;
+}
+
+int pplx_a2a_world_abandon_step(pplx_a2a_world_t *w, uint32_t which, uint32_t *dropped_calls) {
+  if (!w) return fail(PPLX_A2A_INVALID_ARGUMENT, "world is NULL");
+  if (which == 0 || (which & ~(uint32_t)(PPLX_A2A_ABANDON_DISPATCH | PPLX_A2A_ABANDON_COMBINE)) != 0)
+    return fail(PPLX_A2A_INVALID_ARGUMENT, "which must be PPLX_A2A_ABANDON_DISPATCH, _COMBINE or both");
+  std::lock_guard<std::mutex> lock(w->mu);
+  uint32_t dropped = 0;
+  // Recorded calls are host state only: nothing of a step reaches the GPU before its last rank
+  // has called.  A split step whose SEND phase has been launched loses what it staged (the next
+  // SEND overwrites it).
+  auto forget = [&](std::vector<uint8_t> &made, uint32_t &count) {
+    if (count < w->dev.R) dropped += count;  // a complete phase has been launched, not recorded
+    std::fill(made.begin(), made.end(), 0);
+    count = 0;
+  };
+  if (which & PPLX_A2A_ABANDON_DISPATCH) {
+    dropped += w->n_arrived_dispatch;
+    reset_dispatch_arrivals(*w);
+    if (w->split_ready) {
+      forget(w->dsend, w->n_dsend);
+      forget(w->drecv, w->n_drecv);
+    }
+  }
+  if (which & PPLX_A2A_ABANDON_COMBINE) {
+    dropped += w->n_arrived_combine;
+    reset_combine_arrivals(*w);
+    if (w->split_ready) {
+      forget(w->csend, w->n_csend);
+      forget(w->crecv, w->n_crecv);
+    }
+  }
+  if (dropped_calls) *dropped_calls = dropped;
+  return PPLX_A2A_OK;
+}
+
 int pplx_a2a_world_reserve_split(pplx_a2a_world_t *w, uint32_t expert_y_elem_bytes) {
   if (!w) return fail(PPLX_A2A_INVALID_ARGUMENT, "world is NULL");
   std::lock_guard<std::mutex> lock(w->mu);
@@ -974,6 +1041,17 @@ int pplx_a2a_static_step(const pplx_a2a_config_t *cfg, int device,
     return fail(PPLX_A2A_INVALID_ARGUMENT, "device %d out of range (%d visible)", device, n_dev);
   DeviceScope scope(device);
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", device);
+  // The first call on a device looks the array up (which may load the code object) and asks the
+  // device for its LDS size: neither belongs into a stream capture.
+  if (!static_scratch_known(device)) {
+    unsigned long long session = 0;
+    st = capture_session(stream, &session);
+    if (st) return st;
+    if (session != 0)
+      return fail(PPLX_A2A_INVALID_STATE,
+                  "the first pplx_a2a_static_step on a device sets the library up and cannot be captured: make "
+                  "one call outside the capture (or create a world on the device) first");
+  }
   d.lds_per_cu = lds_per_cu_of(device);
   void *base = nullptr;
   LAUNCH_TRY(static_scratch_address(device, &base));

@@ -167,6 +167,8 @@ constexpr uint64_t kWriteThroughMaxBytes = 192ull << 20;
 constexpr size_t kStaticScratchBytes = 8u << 20;
 // Address of the calling thread's current device's copy (looked up once per device).
 int static_scratch_address(int device, void **out);
+// True once static_scratch_address has succeeded for `device`.
+bool static_scratch_known(int device);
 
 struct BindDispatchBatch {
   uint32_t first, count;

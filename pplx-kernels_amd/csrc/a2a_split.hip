@@ -218,8 +218,13 @@ __global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, Sp
   const uint32_t v = (uint32_t)(pair / w.K);
   const uint32_t g = v / w.M;
   const uint32_t t = v - g * w.M;
-  if (t >= combine_rank_tokens(w, tab.at(g * w.dp))) return;
-  const uint32_t e = as_global(sp.gexp)[pair];
+  const CombineRank &head = tab.at(g * w.dp);
+  if (t >= combine_rank_tokens(w, head)) return;
+  // The pair's expert comes from this call's own indices, as in combine_gather: the routing
+  // tables of split mode's dispatch SEND say nothing about a step that was dispatched in one
+  // call.  The slot map alone says whether the pair has a row (a repeated or unknown expert
+  // has none), whichever form of dispatch wrote it.
+  const uint32_t e = as_global(head.indices)[pair - (uint64_t)g * w.M * w.K];
   const uint32_t slot = as_global(w.slot_map)[pair];
   if (e >= w.E || slot == kInvalidSlot) return;
   const CombineRank &own = tab.at(e / w.L);

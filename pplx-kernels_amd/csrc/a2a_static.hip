@@ -42,4 +42,10 @@ int static_scratch_address(int device, void **out) {
   return (int)hipSuccess;
 }
 
+bool static_scratch_known(int device) {
+  if (device < 0 || device >= kMaxDevices) return false;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  return g_scratch_of_device[device] != nullptr;
+}
+
 }  // namespace pplx_amd

@@ -26,7 +26,7 @@ from typing import Any
 import torch
 
 from . import ops
-from .ops import _ops
+from .ops import _C, _ops
 
 
 class AllToAll:
@@ -79,9 +79,9 @@ class AllToAll:
             assert out_expert_x_scale is None
             assert dp_x_scale is None
         # Under torch.compile the call goes through the registered op (what the reference always
-        # does, src/pplx_kernels/all_to_all.py:47-59) so that it traces; an eager call skips the
-        # op dispatcher, which is a fifth of its host time, and runs the op's implementation.
-        fn = self._dispatch_fn if torch.compiler.is_compiling() else ops._dispatch
+        # does, src/pplx_kernels/all_to_all.py:47-59) so that it traces; an eager call enters the
+        # op's implementation directly, without the dispatcher's boxing of ten arguments.
+        fn = self._dispatch_fn if torch.compiler.is_compiling() else _C.dispatch
         fn(
             self._ptr,
             out_expert_num_tokens,
@@ -108,7 +108,7 @@ class AllToAll:
         """``out_tokens[t] = sum_k weights[t, k] * expert_y[slot of (t, k)]`` for
         ``t < bound_m``, fp32 accumulation in pick order; later rows are left as they are."""
         assert self._ptr is not None
-        fn = self._combine_fn if torch.compiler.is_compiling() else ops._combine
+        fn = self._combine_fn if torch.compiler.is_compiling() else _C.combine
         fn(
             self._ptr,
             out_tokens,

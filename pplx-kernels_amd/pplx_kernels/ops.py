@@ -1,17 +1,19 @@
-"""Loads ``libpplx_kernels.so`` (the C ABI of ``include/pplx_a2a.h``) and registers the
-``torch.ops.pplx_kernels`` operators with the reference's schemas.
+"""Loads the native libraries of the package and exposes their entry points.
 
-Mirrors the reference's binding layer: the loader of ``src/pplx_kernels/ops.py:8-16`` and
-the op registration + tensor checks of ``csrc/bindings/all_to_all_ops.cpp:19-24,110-196,
-238-311,329-391``.  Differences that follow from the single-GPU loopback:
+Two shared objects sit next to this file (built by ``make -C pplx-kernels_amd/csrc``):
 
-* the library has no torch types in its interface, so the tensor checks and the stride
-  extraction happen here and raw pointers cross a ctypes call;
-* ``all_to_all_intranode_create`` resolves ``group_name`` to a process-local *world* that
-  owns the state shared by all simulated ranks (the reference resolves a c10d process group
-  and exchanges IPC handles, ``csrc/bindings/all_to_all_ops.cpp:79-106``);
-* a missing or unloadable library is an ``ImportError`` when an op is first used, never a
-  silent fallback.
+* ``_C.so`` -- the torch operator layer (``csrc/torch_ops.cpp``), the counterpart of the
+  reference's ``csrc/bindings/all_to_all_ops.cpp`` + ``bindings.cpp``.  Importing it registers
+  ``torch.ops.pplx_kernels.all_to_all_{intranode,internode}_{create,dispatch,combine}`` and
+  ``all_to_all_destroy`` with the reference's schemas (``all_to_all_ops.cpp:329-391``), as the
+  reference's loader does with ``torch.ops.load_library`` (``src/pplx_kernels/ops.py:8-16``);
+  its module functions ``_C.dispatch`` / ``_C.combine`` are the same code without the op
+  dispatcher, which ``AllToAll`` uses for eager calls.
+* ``libpplx_kernels.so`` -- the C ABI of ``include/pplx_a2a.h`` (kernels + host layer, no
+  torch types), which ``_C.so`` links against and which ``LoopbackWorld`` and the tests also
+  reach through ``ctypes``.
+
+A missing or unloadable library is an ``ImportError``: there is no fallback implementation.
 """
 
 from __future__ import annotations
@@ -45,11 +47,14 @@ EXPORTED_SYMBOLS = (
     "pplx_a2a_destroy",
     "pplx_a2a_num_experts_per_token",
     "pplx_a2a_rank",
+    "pplx_a2a_world_of",
     "pplx_a2a_dispatch",
     "pplx_a2a_combine",
     "pplx_a2a_world_dispatch",
     "pplx_a2a_world_combine",
     "pplx_a2a_static_step",
+    "pplx_a2a_world_recorded_calls",
+    "pplx_a2a_world_abandon_step",
     "pplx_a2a_world_reserve_split",
     "pplx_a2a_world_faults",
     "pplx_a2a_graph_begin_capture",
@@ -159,6 +164,10 @@ def load_library() -> ctypes.CDLL:
         lib.pplx_a2a_static_step.argtypes = [
             ctypes.POINTER(Config), i32, ctypes.POINTER(DispatchArgs), ctypes.POINTER(CombineArgs), vp, vp,
         ]  # fmt: skip
+        lib.pplx_a2a_world_of.argtypes = [vp]
+        lib.pplx_a2a_world_of.restype = vp
+        lib.pplx_a2a_world_recorded_calls.argtypes = [vp, i32, i32, ctypes.POINTER(u32)]
+        lib.pplx_a2a_world_abandon_step.argtypes = [vp, u32, ctypes.POINTER(u32)]
         lib.pplx_a2a_world_reserve_split.argtypes = [vp, u32]
         lib.pplx_a2a_world_faults.argtypes = [vp, vp, ctypes.POINTER(u32)]
         lib.pplx_a2a_graph_begin_capture.argtypes = [vp]
@@ -184,206 +193,56 @@ def check_status(status: int) -> None:
 
 
 # ---------------------------------------------------------------------------
-# Worlds: group_name -> the owner of all simulated ranks' shared state.
+# The torch operator layer
 # ---------------------------------------------------------------------------
-class _World:
-    def __init__(self, key, cfg_tuple, ptr):
-        self.key = key
-        self.cfg = cfg_tuple
-        self.ptr = ptr
-        self.handles: set[int] = set()
-        self.experts_per_token = cfg_tuple[2]
-        self.world_size = cfg_tuple[3]
-        # A step's kernels are enqueued by the last rank to call, so the tensors of the
-        # ranks that called earlier are kept alive until then: a temporary such as
-        # ``x.to(device)`` must not go back to the caching allocator before it is read.
-        # (the same holds for every phase of split mode, which is collective as well)
-        self.pending: dict[str, dict[int, tuple]] = {
-            f"{op}{mode}": {} for op in ("dispatch", "combine") for mode in (SPLIT_NONE, SPLIT_SEND, SPLIT_RECV)
-        }
-        # Widest expert_y element (bytes) that split-mode staging has been reserved for;
-        # -1 = none reserved yet.
-        self.split_reserved = -1
+_BINDING_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_C.so")
+try:
+    from . import _C  # noqa: E402  (registers torch.ops.pplx_kernels)
+except ImportError as exc:
+    raise ImportError(
+        f"cannot load {_BINDING_PATH} ({exc}): build it with `make -C pplx-kernels_amd/csrc` "
+        "(or __graft_entry__.build()); there is no fallback implementation"
+    ) from exc
 
-    def hold(self, kind: str, fptr: int, tensors: tuple) -> None:
-        held = self.pending[kind]
-        held[fptr] = tensors
-        if len(held) >= self.world_size:
-            held.clear()
+_ops = torch.ops.pplx_kernels
+# Interpreter exit: release every world while Python and the HIP runtime are still up;
+# AllToAll.__del__ finds nothing left to do afterwards.
+atexit.register(_C.destroy_all)
 
-    def release(self, fptr: int) -> None:
-        """A handle that is destroyed in the middle of a step takes its half-made calls along."""
-        for held in self.pending.values():
-            held.pop(fptr, None)
+ABANDON_DISPATCH, ABANDON_COMBINE = 1, 2
 
 
-_worlds: dict[str, _World] = {}
-_handle_world: dict[int, _World] = {}
-_registry_lock = threading.Lock()
+class WorldRef:
+    """The world a rank handle is attached to: ``ptr`` is its ``pplx_a2a_world_t *``."""
+
+    def __init__(self, fptr: int) -> None:
+        self.fptr = fptr
+        self.ptr = _C.world_ptr(fptr)
 
 
-def world_of(fptr: int) -> _World:
-    return _handle_world[fptr]
+def world_of(fptr: int) -> WorldRef:
+    return WorldRef(fptr)
 
 
-def _create(
-    transport: str,
-    max_num_tokens: int,
-    num_experts: int,
-    experts_per_token: int,
-    rank: int,
-    world_size: int,
-    dp_size: int,
-    hidden_dim: int,
-    hidden_dim_bytes: int,
-    hidden_dim_scale_bytes: int,
-    group_name: str,
-) -> int:
-    lib = load_library()
-    cfg_tuple = (
-        max_num_tokens,
-        num_experts,
-        experts_per_token,
-        world_size,
-        dp_size,
-        hidden_dim,
-        hidden_dim_bytes,
-        hidden_dim_scale_bytes,
-    )
-    key = f"{transport}:{group_name}"
-    with _registry_lock:
-        world = _worlds.get(key)
-        if world is not None and world.cfg != cfg_tuple:
-            raise RuntimeError(
-                f"pplx_kernels: group '{group_name}' already holds a world with a different "
-                f"configuration {world.cfg}; destroy its ranks first or use another group_name"
-            )
-        if world is None:
-            if min(cfg_tuple) < 0 or world_size <= 0 or dp_size <= 0:
-                raise RuntimeError("pplx_kernels: invalid argument: negative or zero size")
-            cfg = Config(*cfg_tuple)
-            ptr = ctypes.c_void_p()
-            device = torch.cuda.current_device() if torch.cuda.is_available() else 0
-            check_status(lib.pplx_a2a_world_create(ctypes.byref(cfg), device, ctypes.byref(ptr)))
-            world = _World(key, cfg_tuple, ptr.value)
-            _worlds[key] = world
-        if rank < 0:
-            raise RuntimeError("pplx_kernels: invalid argument: negative rank")
-        handle = ctypes.c_void_p()
-        try:
-            check_status(lib.pplx_a2a_create(world.ptr, rank, ctypes.byref(handle)))
-        except RuntimeError:
-            if not world.handles:
-                lib.pplx_a2a_world_destroy(world.ptr)
-                del _worlds[key]
-            raise
-        world.handles.add(handle.value)
-        _handle_world[handle.value] = world
-        return handle.value
-
-
-def _destroy(fptr: int) -> None:
-    lib = load_library()
-    with _registry_lock:
-        world = _handle_world.pop(fptr, None)
-        if world is None:
-            raise RuntimeError(f"pplx_kernels: unknown all-to-all handle {fptr:#x}")
-        check_status(lib.pplx_a2a_destroy(fptr))
-        world.handles.discard(fptr)
-        world.release(fptr)
-        if not world.handles:
-            check_status(lib.pplx_a2a_world_destroy(world.ptr))
-            _worlds.pop(world.key, None)
-
-
-def _destroy_all() -> None:
-    """Interpreter exit: release every world while Python and the HIP runtime are still up;
-    AllToAll.__del__ finds nothing left to do afterwards."""
-    try:
-        lib = load_library()
-    except ImportError:
-        return
-    with _registry_lock:
-        for fptr in list(_handle_world):
-            lib.pplx_a2a_destroy(fptr)
-        _handle_world.clear()
-        for world in list(_worlds.values()):
-            lib.pplx_a2a_world_destroy(world.ptr)
-        _worlds.clear()
-
-
-atexit.register(_destroy_all)
-
-
-def reserve_split(world: _World, expert_y_elem_bytes: int) -> None:
+def reserve_split(world: WorldRef, expert_y_elem_bytes: int) -> None:
     """Split send / recv calls go through staging that the library never allocates inside
-    dispatch / combine.  The reference's callers do not know of it, so the binding reserves it
-    the first time a rank splits a call (and widens it for a wider ``expert_y`` dtype); like
-    any allocation this synchronises and cannot happen under stream capture: run one eager
-    step before capturing split calls, or call this up front."""
-    if world.split_reserved >= expert_y_elem_bytes:
-        return
-    check_status(load_library().pplx_a2a_world_reserve_split(world.ptr, expert_y_elem_bytes))
-    world.split_reserved = expert_y_elem_bytes
+    dispatch / combine.  The reference's callers do not know of it, so the operator layer
+    reserves it the first time a rank splits a call (and widens it for a wider ``expert_y``
+    dtype); like any allocation this synchronises and cannot happen under stream capture: run
+    one eager step before capturing split calls, or call this up front with the widest
+    ``expert_y`` element (a world whose split calls have been captured cannot widen any more)."""
+    _C.reserve_split(world.fptr, expert_y_elem_bytes)
+
+
+def abandon_step(fptr: int, which: int = ABANDON_DISPATCH | ABANDON_COMBINE) -> int:
+    """Drops the calls recorded for the step being assembled in the world of ``fptr`` (and the
+    tensors kept alive for them); returns how many calls were dropped.  The operator layer does
+    this by itself when a rank's arguments are refused after other ranks have called."""
+    return _C.abandon_step(fptr, which)
 
 
 def is_live(fptr: int) -> bool:
-    return fptr in _handle_world
-
-
-def _create_intranode(
-    max_num_tokens: int,
-    num_experts: int,
-    experts_per_token: int,
-    rank: int,
-    world_size: int,
-    dp_size: int,
-    hidden_dim: int,
-    hidden_dim_bytes: int,
-    hidden_dim_scale_bytes: int,
-    group_name: str,
-) -> int:
-    return _create(
-        "intranode",
-        max_num_tokens,
-        num_experts,
-        experts_per_token,
-        rank,
-        world_size,
-        dp_size,
-        hidden_dim,
-        hidden_dim_bytes,
-        hidden_dim_scale_bytes,
-        group_name,
-    )
-
-
-def _create_internode(
-    max_num_tokens: int,
-    num_experts: int,
-    experts_per_token: int,
-    rank: int,
-    world_size: int,
-    dp_size: int,
-    hidden_dim: int,
-    hidden_dim_bytes: int,
-    hidden_dim_scale_bytes: int,
-) -> int:
-    # One HBM has no second transport: the internode constructor attaches to a
-    # loopback world of its own and runs the same kernels.
-    return _create(
-        "internode",
-        max_num_tokens,
-        num_experts,
-        experts_per_token,
-        rank,
-        world_size,
-        dp_size,
-        hidden_dim,
-        hidden_dim_bytes,
-        hidden_dim_scale_bytes,
-        "default",
-    )
+    return _C.is_live(fptr)
 
 
 # ---------------------------------------------------------------------------
@@ -524,104 +383,3 @@ def pack_combine_args(
     a.m = indices.size(0)
     a.bound_m = bound_m.data_ptr() if bound_m is not None else None
     return a
-
-
-def _current_stream(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
-
-
-def _dispatch(
-    fptr: int,
-    out_expert_num_tokens: torch.Tensor,
-    out_expert_x: torch.Tensor,
-    out_expert_x_scale: torch.Tensor | None,
-    dp_x: torch.Tensor,
-    dp_x_scale: torch.Tensor | None,
-    indices: torch.Tensor,
-    bound_m: torch.Tensor | None,
-    do_send: bool,
-    do_recv: bool,
-) -> None:
-    lib = load_library()
-    world = _handle_world.get(fptr)
-    if world is None:
-        raise RuntimeError("pplx_kernels: invalid state: the handle has been destroyed")
-    args = pack_dispatch_args(
-        world.experts_per_token, out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x,
-        dp_x_scale, indices, bound_m,
-    )  # fmt: skip
-    mode = split_mode(do_send, do_recv)
-    if mode != SPLIT_NONE:
-        reserve_split(world, 0)
-    # The library selects the world's device for the launch and restores the caller's; the
-    # stream is the current one of the tensors' device (csrc/bindings/all_to_all_ops.cpp:163,194).
-    check_status(lib.pplx_a2a_dispatch(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    world.hold(
-        f"dispatch{mode}",
-        fptr,
-        (out_expert_num_tokens, out_expert_x, out_expert_x_scale, dp_x, dp_x_scale, indices, bound_m),
-    )
-
-
-def _combine(
-    fptr: int,
-    out_tokens: torch.Tensor,
-    indices: torch.Tensor,
-    weights: torch.Tensor,
-    expert_y: torch.Tensor,
-    bound_m: torch.Tensor | None,
-    do_send: bool,
-    do_recv: bool,
-) -> None:
-    lib = load_library()
-    world = _handle_world.get(fptr)
-    if world is None:
-        raise RuntimeError("pplx_kernels: invalid state: the handle has been destroyed")
-    args = pack_combine_args(out_tokens, indices, weights, expert_y, bound_m)
-    mode = split_mode(do_send, do_recv)
-    if mode != SPLIT_NONE:
-        reserve_split(world, expert_y.element_size())
-    check_status(lib.pplx_a2a_combine(fptr, ctypes.byref(args), mode, _current_stream(indices)))
-    world.hold(f"combine{mode}", fptr, (out_tokens, indices, weights, expert_y, bound_m))
-
-
-def _fake_dispatch(*args, **kwargs) -> None:
-    """Meta kernel: traces as a no-op (csrc/bindings/all_to_all_ops.cpp:198-209)."""
-
-
-def _fake_combine(*args, **kwargs) -> None:
-    """Meta kernel: traces as a no-op (csrc/bindings/all_to_all_ops.cpp:313-322)."""
-
-
-# ---------------------------------------------------------------------------
-# torch.ops.pplx_kernels registration (csrc/bindings/all_to_all_ops.cpp:329-391)
-# ---------------------------------------------------------------------------
-_CREATE_ARGS = (
-    "int max_num_tokens, int num_experts, int experts_per_token, int rank, int world_size, "
-    "int dp_size, int hidden_dim, int hidden_dim_bytes, int hidden_dim_scale_bytes"
-)
-_DISPATCH_SCHEMA = (
-    "(int fptr, Tensor! out_expert_num_tokens, Tensor! out_expert_x, Tensor!? out_expert_x_scale, "
-    "Tensor dp_x, Tensor? dp_x_scale, Tensor indices, Tensor? bound_m, bool do_send, bool do_recv) -> ()"
-)
-_COMBINE_SCHEMA = (
-    "(int fptr, Tensor! out_tokens, Tensor indices, Tensor weights, Tensor expert_y, "
-    "Tensor? bound_m, bool do_send, bool do_recv) -> ()"
-)
-
-_torch_lib = torch.library.Library("pplx_kernels", "DEF")
-_torch_lib.define("all_to_all_destroy(int fptr) -> ()")
-_torch_lib.impl("all_to_all_destroy", _destroy, "CompositeExplicitAutograd")
-_torch_lib.define(f"all_to_all_intranode_create({_CREATE_ARGS}, str group_name) -> int")
-_torch_lib.impl("all_to_all_intranode_create", _create_intranode, "CompositeExplicitAutograd")
-_torch_lib.define(f"all_to_all_internode_create({_CREATE_ARGS}) -> int")
-_torch_lib.impl("all_to_all_internode_create", _create_internode, "CompositeExplicitAutograd")
-for _transport in ("intranode", "internode"):
-    _torch_lib.define(f"all_to_all_{_transport}_dispatch{_DISPATCH_SCHEMA}")
-    _torch_lib.impl(f"all_to_all_{_transport}_dispatch", _dispatch, "CUDA")
-    _torch_lib.impl(f"all_to_all_{_transport}_dispatch", _fake_dispatch, "Meta")
-    _torch_lib.define(f"all_to_all_{_transport}_combine{_COMBINE_SCHEMA}")
-    _torch_lib.impl(f"all_to_all_{_transport}_combine", _combine, "CUDA")
-    _torch_lib.impl(f"all_to_all_{_transport}_combine", _fake_combine, "Meta")
-
-_ops = torch.ops.pplx_kernels

@@ -742,6 +742,41 @@ def test_split_order_is_enforced():
         a.destroy()
 
 
+def test_split_combine_after_a_one_call_dispatch():
+    """combine SEND / RECV does not care how the step was dispatched (the reference's combine
+    reads what its own dispatch recorded, whichever mode that ran in): a split step with one
+    routing, then a one-call dispatch with another routing followed by a split combine."""
+    spec = _small_spec(name="split-mixed", in_dtype=FP8, hidden_dim=1024)
+    ranks = _make_ranks(spec, "split-mixed")
+    R = spec.world_size
+    first = DeviceStep(spec, generate(spec, seed=21))
+    for r in range(R):
+        ranks[r].dispatch(**_dispatch_kw(first, r), do_send=True, do_recv=False)
+    for r in range(R):
+        ranks[r].dispatch(**_dispatch_kw(first, r), do_send=False, do_recv=True)
+    expected = check_dispatch_against_oracle(first)
+    first.expert_y_all.normal_()
+    for r in range(R):
+        ranks[r].combine(**_combine_kw(first, r), do_send=True, do_recv=False)
+    for r in range(R):
+        ranks[r].combine(**_combine_kw(first, r), do_send=False, do_recv=True)
+    check_combine_against_oracle(first, expected.slot_map)
+
+    second = DeviceStep(spec, generate(spec, seed=22))
+    assert any(not torch.equal(a.indices, b.indices) for a, b in zip(first.groups, second.groups))
+    for r in range(R):
+        ranks[r].dispatch(**_dispatch_kw(second, r))
+    expected = check_dispatch_against_oracle(second)
+    second.expert_y_all.normal_()
+    for r in range(R):
+        ranks[r].combine(**_combine_kw(second, r), do_send=True, do_recv=False)
+    for r in reversed(range(R)):
+        ranks[r].combine(**_combine_kw(second, r), do_send=False, do_recv=True)
+    check_combine_against_oracle(second, expected.slot_map)
+    for a in ranks:
+        a.destroy()
+
+
 # ---------------------------------------------------------------------------
 # hipGraph replay (decode shape)
 # ---------------------------------------------------------------------------

@@ -27,7 +27,7 @@ def declared_symbols() -> list[str]:
 def test_library_exports_every_declared_symbol():
     lib = ops.load_library()
     names = declared_symbols()
-    assert len(names) >= 19
+    assert len(names) >= 23
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in include/pplx_a2a.h but not exported"
     assert sorted(ops.EXPORTED_SYMBOLS) == names
@@ -53,6 +53,15 @@ def test_library_is_built_from_the_sources_in_the_tree():
     assert ops.load_library().pplx_a2a_build_id().decode() == h.hexdigest()[:16], (
         "libpplx_kernels.so is stale: run `make -C pplx-kernels_amd/csrc`"
     )
+
+
+def test_operator_layer_is_built_from_the_sources_in_the_tree():
+    import hashlib
+
+    h = hashlib.sha256()
+    h.update(open(os.path.join(ROOT, "pplx-kernels_amd", "csrc", "torch_ops.cpp"), "rb").read())
+    h.update(open(HEADER, "rb").read())
+    assert ops._C.build_id() == h.hexdigest()[:16], "pplx_kernels/_C.so is stale: run `make -C pplx-kernels_amd/csrc`"
 
 
 def test_ctypes_structs_match_the_header_layout():
@@ -116,6 +125,9 @@ def test_null_arguments_are_status_codes_not_crashes():
     assert lib.pplx_a2a_world_dispatch(None, None, None) == 1
     assert lib.pplx_a2a_world_faults(None, None, None) == 1
     assert lib.pplx_a2a_world_reserve_split(None, 2) == 1
+    assert lib.pplx_a2a_world_abandon_step(None, 3, None) == 1
+    assert lib.pplx_a2a_world_recorded_calls(None, 0, 0, None) == 1
+    assert lib.pplx_a2a_world_of(None) is None
     assert lib.pplx_a2a_graph_launch(None, None) == 1
     assert lib.pplx_a2a_destroy(None) == 0 and lib.pplx_a2a_world_destroy(None) == 0
     assert lib.pplx_a2a_graph_destroy(None) == 0
