@@ -212,6 +212,10 @@ void fill_geometry(const pplx_a2a_config_t &cfg, WorldDev &d) {
   d.H = (uint32_t)cfg.hidden_dim;
   d.Hb = (uint32_t)cfg.hidden_dim_bytes;
   d.S = (uint32_t)(cfg.hidden_dim_scale_bytes / 4);
+  d.by_M = make_fast_div(d.M);
+  d.by_dp = make_fast_div(d.dp);
+  d.by_L = make_fast_div(d.L);
+  d.by_K = make_fast_div(d.K);
   // Routing tiles of a whole step: small enough that a step has a few hundred of them (a tile
   // is one workgroup, and routing is a chain of short launches that only parallelism shortens),
   // at most 16 chunks of 64 tokens, and such that the LDS tables fit 64 KiB.

@@ -92,15 +92,15 @@ __device__ __forceinline__ void gather_group(f32x8 (&acc)[VPL], uint64_t row_of_
 // row) and takes the picks KB at a time, so KB * VPL row loads per lane are in flight: few
 // picks read long pieces of their rows, many picks shorter ones.
 template <typename T, typename U, class CT, int KB, int VPL>
-__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments,
+__global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments, FastDiv by_segments,
                                                       uint32_t first_rank, uint32_t rank_count,
                                                       const uint8_t *stage_y, uint64_t stage_row_bytes) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
                                                        threadIdx.x / kWave);
-  const uint32_t token = wave / segments;
+  const uint32_t token = fast_div(wave, by_segments);
   const uint32_t segment = wave - token * segments;
-  const uint32_t r_local = token / w.M;
+  const uint32_t r_local = group_of(w, token);
   const uint32_t t = token - r_local * w.M;
   if (r_local >= rank_count) return;
   const uint32_t r = first_rank + r_local;
@@ -112,19 +112,19 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
   float weight = 0.f;
   if (lane < w.K) {
     const uint32_t e = as_global(c.indices)[(size_t)t * w.K + lane];
-    const uint32_t slot = as_global(w.slot_map)[((size_t)(r / w.dp) * w.M + t) * w.K + lane];
+    const uint32_t slot = as_global(w.slot_map)[((size_t)fast_div(r, w.by_dp) * w.M + t) * w.K + lane];
     weight = as_global(c.weights)[(int64_t)t * c.w_stride_row + lane];
     if (CT::kStaged) {
       // combine SEND left the row of (token, pick) in the staging area.
       if (e < w.E && slot != kInvalidSlot) {
         row = reinterpret_cast<uint64_t>(stage_y) +
-              (((uint64_t)(r / w.dp) * w.M + t) * w.K + lane) * stage_row_bytes;
+              (((uint64_t)fast_div(r, w.by_dp) * w.M + t) * w.K + lane) * stage_row_bytes;
       }
     } else if (e < w.E && slot != kInvalidSlot) {
-      const CombineRank &owner = tab.at(e / w.L);
+      const CombineRank &owner = tab.at(owner_of(w, e));
       if (slot < owner.y_rows) {
         row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
-                                         (int64_t)(e % w.L) * owner.y_stride_expert +
+                                         (int64_t)local_of(w, e) * owner.y_stride_expert +
                                          (int64_t)slot * owner.y_stride_row);
       } else if (segment == 0) {
         atomicOr(w.faults, kFaultBadSlot);
@@ -182,7 +182,8 @@ int launch_combine_v(const WorldDev &w, const CT &tab, uint32_t first_rank, uint
   const uint32_t segments = (nvec_segments + VPL - 1) / VPL;
   const uint64_t waves = (uint64_t)rank_count * w.M * segments;
   const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
-  hipLaunchKernelGGL((combine_gather<T, U, CT, KB, VPL>), grid, block, 0, s, w, tab, segments, first_rank,
+  hipLaunchKernelGGL((combine_gather<T, U, CT, KB, VPL>), grid, block, 0, s, w, tab, segments,
+                     make_fast_div(segments), first_rank,
                      rank_count, stage_y, stage_row_bytes);
   return (int)hipGetLastError();
 }

@@ -163,6 +163,16 @@ __device__ __forceinline__ uint64_t read_lane64(uint64_t v, uint32_t src_lane) {
          (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, (int)src_lane);
 }
 
+// Virtual token v = g * M + t.
+__device__ __forceinline__ uint32_t group_of(const WorldDev &w, uint32_t v) { return fast_div(v, w.by_M); }
+// The member of DP group g that sends token t (csrc/all_to_all/intranode_dispatch.cu:97): g * dp + t % dp.
+__device__ __forceinline__ uint32_t sender_of(const WorldDev &w, uint32_t g, uint32_t t) {
+  return g * w.dp + (t - fast_div(t, w.by_dp) * w.dp);
+}
+// Expert e lives on rank e / L as local expert e % L (csrc/all_to_all/intranode_dispatch.cu:133-134).
+__device__ __forceinline__ uint32_t owner_of(const WorldDev &w, uint32_t e) { return fast_div(e, w.by_L); }
+__device__ __forceinline__ uint32_t local_of(const WorldDev &w, uint32_t e) { return e - fast_div(e, w.by_L) * w.L; }
+
 // Tokens present in DP group g this step: the reference's numSendTokens
 // (csrc/all_to_all/intranode_dispatch.cu:64), clamped to the rows that exist.
 template <class DT>

@@ -21,6 +21,31 @@ constexpr uint32_t kFaultBadSlot = 4u;      // combine slot >= expert_y rows
 constexpr uint32_t kFaultDuplicateExpert = 8u;   // an expert id repeated inside one token was dropped
 constexpr uint32_t kFaultTooManyTokens = 16u;    // bound_m > max_num_tokens (or > rows) was clamped
 
+// Division by a number that is fixed for a launch (tokens per group, experts per rank ...):
+// a multiply-high, a subtract, an add and two shifts instead of the thirty-odd instructions of
+// a 32-bit hardware-less division (Granlund & Montgomery, "Division by invariant integers using
+// multiplication", figure 4.1, N = 32).  Exact for every 32-bit numerator and divisor >= 1.
+struct FastDiv {
+  uint32_t mul;
+  uint32_t shifts;  // sh1 (0 or 1) in bit 0, sh2 from bit 8 up: q = (t + ((n - t) >> sh1)) >> sh2
+};
+inline FastDiv make_fast_div(uint32_t d) {
+  FastDiv f{1u, 0u};
+  if (d <= 1) return f;  // l = 0: q = n
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;  // ceil(log2 d)
+  f.mul = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+  f.shifts = 1u | ((l - 1) << 8);
+  return f;
+}
+#ifdef __HIPCC__
+__host__ __device__
+#endif
+inline uint32_t fast_div(uint32_t n, const FastDiv &f) {
+  const uint32_t t = (uint32_t)(((uint64_t)f.mul * n) >> 32);
+  return (t + ((n - t) >> (f.shifts & 1u))) >> (f.shifts >> 8);
+}
+
 struct alignas(16) DispatchRank {
   int32_t *out_num_tokens;
   int64_t out_num_tokens_stride;
@@ -74,6 +99,7 @@ struct WorldDev {
   uint32_t tile_chunks;  // 64-token chunks per routing tile of a whole-step dispatch
   uint32_t num_tiles;    // ceil(G * M / (64 * tile_chunks))
   uint32_t lds_per_cu;   // bytes of LDS a CU has (0 = unknown): launches use it to cap residency
+  FastDiv by_M, by_dp, by_L, by_K;  // fast_div(n, by_X) == n / X
   DispatchRank *drank;   // [R]
   CombineRank *crank;    // [R]
   uint32_t *tile_cnt;    // [num_tiles][E] tokens routed to e inside a tile; after route_scan the

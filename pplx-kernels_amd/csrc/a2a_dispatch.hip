@@ -55,14 +55,13 @@ __device__ __forceinline__ void scatter_token(const WorldDev &w, const DT &tab, 
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
                                                        threadIdx.x / kWave);
-  const uint32_t v = wave / ksplit;
+  const uint32_t v = wave >> __builtin_ctz(ksplit);  // (ksplit is a power of two)
   const uint32_t part = wave - v * ksplit;
-  const uint32_t g = v / w.M;
+  const uint32_t g = group_of(w, v);
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
   if (t >= dispatch_group_tokens(w, tab, g)) return;
-  // The sender of token t inside its DP group (csrc/all_to_all/intranode_dispatch.cu:97).
-  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  const DispatchRank &src = tab.at(sender_of(w, g, t));
   RowRegs<NV> regs;
   load_row<NV, EXACT>(w, src, t, lane, regs);
   Destination dst;
@@ -112,22 +111,19 @@ struct LdsDispatch {
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
 
-// Reads the picks of virtual tokens [0, v_own_end), one thread per token and PV picks per load
-// (K % PV == 0 and every indices pointer aligned to the vector: the host checks both): those
-// of tokens before v_own go into the LDS histogram, those of the workgroup's own tokens
-// [v_own, v_own_end) into own_e for phase 3.
+// Counts, per expert, the tokens before virtual token v_end that are routed to it, into the LDS
+// histogram `hist`: one thread per token and pass, PV picks per load (K % PV == 0 and every
+// indices pointer aligned to the vector: the host checks both).  Every expert a token names
+// counts once (a repeat inside the token takes no row).
 //
 // The loads of a token (its group's token count and its first two vectors of picks) are
 // unconditional, from a harmless address when the thread has no token, and sit in
 // straight-line code: they are issued together and cost one trip to memory, and the count is
-// applied afterwards.  `between` runs after the loads of the thread's first token have been
-// issued and before they are used: whatever it loads is in flight behind them (a wave's loads
-// complete in order).  The bookkeeping per token is one division: this loop is bound by the
-// ALU, not by memory, when every workgroup of a launch repeats it.
-template <int PV, uint32_t THREADS, class Table, class Between>
-__device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows, uint32_t v_own,
-                                           uint32_t v_own_end, uint32_t *hist, uint32_t *own_e,
-                                           Between &&between) {
+// applied afterwards.  The loads of the next pass are issued before the picks of this one are
+// counted, so a step of several passes pays one trip, not one per pass.
+template <int PV, uint32_t THREADS, class Table>
+__device__ __forceinline__ void count_earlier_picks(const WorldDev &w, const Table &rows, uint32_t v_end,
+                                                    uint32_t *hist) {
   typedef PickVector<PV> Vec;
   typedef typename Vec::type vec_t;
   const uint32_t vectors = w.K / PV;
@@ -140,11 +136,11 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
   };
   auto issue = [&](uint32_t v) {
     Fetch f;
-    const bool in_range = v < v_own_end;
-    const uint32_t g = in_range ? v / w.M : 0;
+    const bool in_range = v < v_end;
+    const uint32_t g = in_range ? group_of(w, v) : 0;
     f.t = in_range ? v - g * w.M : 0;
     const DispatchRank &head = rows.at(g * w.dp);
-    const DispatchRank &src = w.dp == 1 ? head : rows.at(g * w.dp + f.t % w.dp);
+    const DispatchRank &src = w.dp == 1 ? head : rows.at(sender_of(w, g, f.t));
     f.valid = in_range && f.t < src.m && f.t < head.m;
     const bool bounded = f.valid && head.bound_m != nullptr;
     const uint32_t loaded_n = *as_global(bounded ? head.bound_m : w.faults);
@@ -154,63 +150,60 @@ __device__ __forceinline__ void read_picks(const WorldDev &w, const Table &rows,
     f.n = bounded ? loaded_n : head.m;
     return f;
   };
-  auto place = [&](uint32_t v, uint32_t j, vec_t a, vec_t b, const Fetch &f) {
+  auto place = [&](uint32_t j, vec_t a, vec_t b, const Fetch &f) {
     const bool second = j + 1 < vectors;
-    if (v >= v_own) {
-      uint32_t *keep = own_e + (v - v_own) * w.K + j * PV;
+    // The picks of this call are compared in registers; those of earlier calls for the same
+    // token (top-k beyond two vectors) are read again.
+    uint32_t e[2 * PV];
 #pragma unroll
-      for (int u = 0; u < PV; ++u) keep[u] = Vec::at(a, u);
+    for (int u = 0; u < PV; ++u) {
+      e[u] = Vec::at(a, u);
+      e[PV + u] = second ? Vec::at(b, u) : w.E;
+    }
 #pragma unroll
-      for (int u = 0; u < PV; ++u) {
-        if (second) keep[PV + u] = Vec::at(b, u);
+    for (int u = 0; u < 2 * PV; ++u) {
+      bool counts = e[u] < w.E;
+#pragma unroll
+      for (int p = 0; p < u; ++p) counts = counts && e[p] != e[u];
+      if (counts && j != 0) {
+        const PPLX_GLOBAL uint32_t *before = reinterpret_cast<const PPLX_GLOBAL uint32_t *>(f.idx);
+        for (uint32_t p = 0; p < j * PV; ++p) counts = counts && before[p] != e[u];
       }
-    } else if (f.t < f.n) {
-      // An earlier token: every expert it names counts once (a repeat takes no row).  The
-      // picks of this call are compared in registers; those of earlier calls for the same
-      // token (top-k beyond two vectors) are read again.
-      uint32_t e[2 * PV];
-#pragma unroll
-      for (int u = 0; u < PV; ++u) {
-        e[u] = Vec::at(a, u);
-        e[PV + u] = second ? Vec::at(b, u) : w.E;
-      }
-#pragma unroll
-      for (int u = 0; u < 2 * PV; ++u) {
-        bool counts = e[u] < w.E;
-#pragma unroll
-        for (int p = 0; p < u; ++p) counts = counts && e[p] != e[u];
-        if (counts && j != 0) {
-          const PPLX_GLOBAL uint32_t *before = reinterpret_cast<const PPLX_GLOBAL uint32_t *>(f.idx);
-          for (uint32_t p = 0; p < j * PV; ++p) counts = counts && before[p] != e[u];
-        }
-        if (counts) atomicAdd(&hist[e[u]], 1u);
-      }
+      if (counts) atomicAdd(&hist[e[u]], 1u);
     }
   };
-  auto consume = [&](uint32_t v, const Fetch &f) {
-    if (!f.valid) return;
-    place(v, 0, f.a, f.b, f);
-    for (uint32_t j = 2; j < vectors; j += 2) place(v, j, f.idx[j], f.idx[j + 1 < vectors ? j + 1 : j], f);
+  auto consume = [&](const Fetch &f) {
+    if (!f.valid || f.t >= f.n) return;
+    place(0, f.a, f.b, f);
+    for (uint32_t j = 2; j < vectors; j += 2) place(j, f.idx[j], f.idx[j + 1 < vectors ? j + 1 : j], f);
   };
 
-  const Fetch first = issue(threadIdx.x);
-  between();
-  consume(threadIdx.x, first);
-  for (uint32_t v = threadIdx.x + THREADS; v < v_own_end; v += THREADS) consume(v, issue(v));
+  Fetch current = issue(threadIdx.x);
+  for (uint32_t v = threadIdx.x + THREADS; v < v_end; v += THREADS) {
+    const Fetch next = issue(v);
+    consume(current);
+    current = next;
+  }
+  consume(current);
 }
 
 // Small steps: one launch does routing and scatter.  A workgroup owns tokens_per_block
-// consecutive virtual tokens and their tokens_per_block * K picks, one thread per pick.
-//   0. a rank table that came inline is copied from the kernel arguments into LDS with loads
-//      that depend on nothing, so every later lookup is an LDS read and not another trip to
-//      memory behind the one that fetches the geometry;
-//   1. index arithmetic for the wave's token and the thread's pick;
-//   2. the workgroup reads the picks of all tokens up to and including its own and counts, per
-//      expert, those of the tokens before its own (every workgroup repeats this over the
-//      indices, which are a few KiB in L2); then every wave issues the loads of its token's
-//      row, which is needed only in phase 4;
-//   3. the pick threads take their slots token by token out of the LDS counters, resolve the
-//      destination rows once for the workgroup and leave them in LDS;
+// consecutive virtual tokens; each of them belongs to one wave (or to ksplit waves that share
+// its picks), and lane k of such a row wave is the token's pick k.
+//   0. the rank table (world_size rows of it) is copied from the kernel arguments into LDS with
+//      loads that depend on nothing, so every later lookup is an LDS read and not another trip
+//      to memory behind the one that fetches the geometry;
+//   1. one batch of small loads: every thread fetches the picks of one token before the
+//      workgroup's own (and its group's token count), the row waves their own picks;
+//   2. the picks of the earlier tokens are counted per expert in an LDS histogram (every
+//      workgroup repeats this over the indices, which are a few KiB in L2); the row waves mark
+//      their token in a per-expert bit mask of the workgroup's own tokens; only then do the row
+//      waves issue the loads of their rows -- the rows are HBM-cold and several KiB per wave,
+//      and the small loads of every wave of the CU would otherwise queue behind them for as
+//      long as the rows take (8 x 128 DSv3 tokens: stores begin 1.6 us earlier this way);
+//   3. behind one barrier a pick's slot is the histogram's count plus the own tokens before
+//      its own that go to the same expert (a popcount of the mask below the token's bit); the
+//      lane resolves its destination row and keeps it in registers;
 //   4. the waves fan their rows out.  The last workgroup has counted everything and writes
 //      out_expert_num_tokens.
 // As dispatch SEND of split mode (`stage` = SplitDev::stage_x) the launch leaves the callers'
@@ -224,19 +217,15 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
   constexpr bool kStaged = DT::kInline;
-  constexpr uint32_t kTableWords = kStaged ? sizeof(DT) / 8 : 0;
+  constexpr uint32_t kRowWords = sizeof(DispatchRank) / 8;
+  const uint32_t table_words = kStaged ? w.R * kRowWords : 0;
   if constexpr (kStaged) {
     const unsigned long long *args = reinterpret_cast<const unsigned long long *>(&tab);
-    for (uint32_t i = threadIdx.x; i < kTableWords; i += kFusedThreads) lds_u64[i] = args[i];
+    for (uint32_t i = threadIdx.x; i < table_words; i += kFusedThreads) lds_u64[i] = args[i];
   }
-  const uint32_t own_pairs = tokens_per_block * w.K;
-  unsigned long long *dst_row = lds_u64 + kTableWords;                         // [own_pairs]
-  unsigned long long *dst_scale = dst_row + own_pairs;                         // [own_pairs]
-  long long *dst_step = reinterpret_cast<long long *>(dst_scale + own_pairs);  // [own_pairs]
-  uint32_t *hist = reinterpret_cast<uint32_t *>(dst_step + own_pairs);         // [E]
-  uint32_t *ntok = hist + w.E;                                                 // [G]
-  uint32_t *own_e = ntok + w.G;                                                // [own_pairs]
-  for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) hist[e] = 0;
+  uint32_t *hist = reinterpret_cast<uint32_t *>(lds_u64 + table_words);  // [E] tokens before the workgroup's own
+  uint32_t *own_mask = hist + w.E;                                       // [E] bit j: own token j goes to e
+  for (uint32_t e = threadIdx.x; e < 2 * w.E; e += kFusedThreads) hist[e] = 0;
   // Orders the zeroing (and the staged table) before the first counter update of any wave.
   __syncthreads();
   const LdsDispatch staged{reinterpret_cast<const DispatchRank *>(lds_u64)};
@@ -247,142 +236,106 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   const uint32_t total = w.G * w.M;
   const uint32_t v0 = blockIdx.x * tokens_per_block;
 
-  // 1a. this wave's token and its row
+  // 1. this wave's token; lane k is its pick k
   const uint32_t lane = lane_id();
   const uint32_t my_wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const uint32_t my_j = my_wave / ksplit;
+  const uint32_t my_j = my_wave >> __builtin_ctz(ksplit);  // (ksplit is a power of two)
   const uint32_t my_part = my_wave - my_j * ksplit;
   const uint32_t my_v = v0 + my_j;
-  const uint32_t my_g = my_v / w.M;
-  const uint32_t my_t = my_v - my_g * w.M;
   const bool my_in_range = my_j < tokens_per_block && my_v < total;
-  const DispatchRank &my_src = rows().at(my_in_range ? my_g * w.dp + my_t % w.dp : 0);
-  const bool my_row_exists = my_in_range && my_t < my_src.m;
-
-  // 1b. this thread's pick (threads beyond own_pairs have none)
-  const uint32_t pick_j = threadIdx.x / w.K;
-  const uint32_t pick_k = threadIdx.x - pick_j * w.K;
-  const uint32_t pick_v = v0 + pick_j;
-  const uint32_t pick_g = pick_v / w.M;
-  const uint32_t pick_t = pick_v - pick_g * w.M;
-  bool pick_exists = threadIdx.x < own_pairs && pick_v < total;
-  if (pick_exists) pick_exists = pick_t < rows().at(pick_g * w.dp + pick_t % w.dp).m;
+  const uint32_t my_g = my_in_range ? group_of(w, my_v) : 0;
+  const uint32_t my_t = my_in_range ? my_v - my_g * w.M : 0;
+  const DispatchRank &my_head = rows().at(my_g * w.dp);
+  const DispatchRank &my_src = w.dp == 1 ? my_head : rows().at(sender_of(w, my_g, my_t));
+  const bool my_row_exists = my_in_range && my_t < my_src.m && my_t < my_head.m;
+  const bool my_bounded = my_row_exists && my_head.bound_m != nullptr;
+  const uint32_t my_loaded_n = *as_global(my_bounded ? my_head.bound_m : w.faults);
+  const bool has_pick = my_row_exists && lane < w.K;
+  const uint32_t my_loaded_e = *as_global(has_pick ? my_src.indices + (size_t)my_t * w.K + lane : w.faults);
 
   // 2. picks of all earlier tokens
-  // (the token count of group `threadIdx.x` is fetched ahead of the picks, in the same batch of
-  // loads, and stored once they have been used: no wave pays for two trips to memory in a row)
-  const bool counts_group = threadIdx.x < w.G;
-  const DispatchRank &counted = rows().at(counts_group ? threadIdx.x * w.dp : 0);
-  const uint32_t *counted_bound = counts_group ? counted.bound_m : nullptr;
-  const uint32_t counted_loaded = *as_global(counted_bound ? counted_bound : w.faults);
-  const uint32_t v_own_end = v0 + tokens_per_block < total ? v0 + tokens_per_block : total;
-  // The row is fetched behind the first picks: a wave's loads complete in order, so the small
-  // loads would otherwise wait behind several KiB of row data.  It is needed in phase 4.
-  RowRegs<NV> regs;
-  auto fetch_row = [&]() {
-    if (my_row_exists) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
-  };
   if (pick_vector == 4) {
-    read_picks<4, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    count_earlier_picks<4, kFusedThreads>(w, rows(), v0, hist);
   } else if (pick_vector == 2) {
-    read_picks<2, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    count_earlier_picks<2, kFusedThreads>(w, rows(), v0, hist);
   } else {
-    read_picks<1, kFusedThreads>(w, rows(), v0, v_own_end, hist, own_e, fetch_row);
+    count_earlier_picks<1, kFusedThreads>(w, rows(), v0, hist);
   }
-  if (counts_group) {
-    const uint32_t asked = counted_bound ? counted_loaded : counted.m;
-    uint32_t n = asked < counted.m ? asked : counted.m;
-    n = n < w.M ? n : w.M;
-    ntok[threadIdx.x] = n;
-    if (n != asked && blockIdx.x == 0) atomicOr(w.faults, kFaultTooManyTokens);
+  // ... and the workgroup's own: a pick that names no expert, or repeats an earlier pick of its
+  // token, has no row.
+  uint32_t my_n = my_bounded ? my_loaded_n : my_head.m;
+  my_n = my_n < w.M ? my_n : w.M;
+  const bool my_live = my_row_exists && my_t < my_n;
+  const uint32_t my_e = has_pick ? my_loaded_e : w.E;
+  bool my_repeats = false;
+  for (uint32_t k = 0; k + 1 < w.K; ++k) {
+    const uint32_t earlier = (uint32_t)__builtin_amdgcn_readlane((int)my_e, (int)k);
+    if (lane > k && earlier == my_e) my_repeats = true;
   }
-  for (uint32_t g = threadIdx.x + kFusedThreads; g < w.G; g += kFusedThreads) {
-    ntok[g] = dispatch_group_tokens(w, rows(), g);
-    if (blockIdx.x == 0 && dispatch_group_overflows(w, rows(), g)) atomicOr(w.faults, kFaultTooManyTokens);
-  }
+  const bool my_pick_has_row = my_live && my_e < w.E && !my_repeats;
+  if (my_pick_has_row && my_part == 0) atomicOr(&own_mask[my_e], 1u << my_j);
+  RowRegs<NV> regs;
+  if (my_live) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
   __syncthreads();
 
-  // 3. own slots, token by token (a pick that repeats an earlier expert of its token takes no
-  // row, so no two threads of a round share a counter), then the destinations
-  const bool pick_live = pick_exists && pick_t < ntok[pick_g];
-  const uint32_t pick_e = pick_exists ? own_e[threadIdx.x] : w.E;
-  bool pick_repeats = false;
-  if (pick_live) {
-    for (uint32_t k = 0; k < pick_k; ++k) pick_repeats = pick_repeats || own_e[threadIdx.x - pick_k + k] == pick_e;
-  }
-  uint32_t pick_slot = kInvalidSlot;
-  // (when all pick threads sit in one wave the hardware keeps its LDS accesses in order by
-  // itself; the fence keeps the compiler from moving them across the rounds)
-  const bool one_wave = own_pairs <= kWave;
-  for (uint32_t j = 0; j < tokens_per_block; ++j) {
-    if (pick_live && pick_j == j && pick_e < w.E && !pick_repeats) {
-      pick_slot = hist[pick_e];
-      hist[pick_e] = pick_slot + 1;
-    }
-    if (one_wave) {
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    } else {
-      __syncthreads();
-    }
-  }
-  if (threadIdx.x < own_pairs) {
-    Destination d;
-    const size_t pair = (size_t)pick_v * w.K + pick_k;
+  // 3. own slots and destinations
+  uint32_t my_slot = kInvalidSlot;
+  if (my_pick_has_row) my_slot = hist[my_e] + __popc(own_mask[my_e] & ((1u << my_j) - 1u));
+  Destination dst;
+  if (my_in_range && lane < w.K) {
+    const size_t pair = (size_t)my_v * w.K + lane;
     if (stage != nullptr) {
       // (whether the slot fits the receiver's rows is for RECV to say)
       const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
-      const bool has_row = pick_live && pick_e < w.E && pick_slot != kInvalidSlot;
-      if (has_row) {
-        d.row = reinterpret_cast<uint64_t>(stage + pair * lay.token_stride);
-        d.scale = d.row + w.Hb;
-        d.scale_step = 1;
-        *global_ptr<uint32_t>(d.row + w.Hb + 4ull * w.S) = pick_t;
+      if (my_pick_has_row) {
+        dst.row = reinterpret_cast<uint64_t>(stage + pair * lay.token_stride);
+        dst.scale = dst.row + w.Hb;
+        dst.scale_step = 1;
+        if (my_part == 0) *global_ptr<uint32_t>(dst.row + w.Hb + 4ull * w.S) = my_t;
       }
-      if (pick_v < total) {
-        as_global(reinterpret_cast<uint32_t *>(stage + lay.gexp_offset))[pair] = has_row ? pick_e : w.E;
+      if (my_part == 0) {
+        as_global(reinterpret_cast<uint32_t *>(stage + lay.gexp_offset))[pair] = my_pick_has_row ? my_e : w.E;
       }
-    } else if (pick_live) {
-      d = resolve_destination(w, rows(), pick_e, pick_slot, true);
+    } else if (my_live) {
+      dst = resolve_destination(w, rows(), my_e, my_slot, my_part == 0);
     }
-    if (pick_live) {
-      as_global(w.slot_map)[pair] = pick_slot;
-      if (pick_e >= w.E) {
+    if (my_live && my_part == 0) {
+      as_global(w.slot_map)[pair] = my_slot;
+      if (my_e >= w.E) {
         atomicOr(w.faults, kFaultBadExpert);
-      } else if (pick_repeats) {
+      } else if (my_repeats) {
         atomicOr(w.faults, kFaultDuplicateExpert);
       }
     }
-    dst_row[threadIdx.x] = d.row;
-    dst_scale[threadIdx.x] = d.scale;
-    dst_step[threadIdx.x] = d.scale_step;
   }
-  __syncthreads();
   if (blockIdx.x == gridDim.x - 1) {
     for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) {
+      const uint32_t rows_of_e = hist[e] + __popc(own_mask[e]);
       if (stage != nullptr) {
         const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
-        as_global(reinterpret_cast<uint32_t *>(stage + lay.gcnt_offset))[e] = hist[e];
+        as_global(reinterpret_cast<uint32_t *>(stage + lay.gcnt_offset))[e] = rows_of_e;
         continue;
       }
-      const DispatchRank &owner = rows().at(e / w.L);
-      as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)hist[e];
+      const DispatchRank &owner = rows().at(owner_of(w, e));
+      as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)rows_of_e;
     }
   }
 
   // 4. fan out
-  if (!my_row_exists || my_t >= ntok[my_g]) return;
-  Destination dst;
-  if (lane < w.K) {
-    dst.row = dst_row[my_j * w.K + lane];
-    dst.scale = dst_scale[my_j * w.K + lane];
-    dst.scale_step = dst_step[my_j * w.K + lane];
+  if (my_live) {
+    const uint32_t k0 = my_part * kper;
+    const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
+    if (write_through) {
+      store_row<NV, EXACT, RowStore::kKeep>(w, my_src, my_t, lane, dst, k0, k1, regs);
+    } else {
+      store_row<NV, EXACT, RowStore::kStream>(w, my_src, my_t, lane, dst, k0, k1, regs);
+    }
   }
-  const uint32_t k0 = my_part * kper;
-  const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
-  if (write_through) {
-    store_row<NV, EXACT, RowStore::kKeep>(w, my_src, my_t, lane, dst, k0, k1, regs);
-  } else {
-    store_row<NV, EXACT, RowStore::kStream>(w, my_src, my_t, lane, dst, k0, k1, regs);
+  // A bound_m beyond the limit is reported once, behind the stores (it costs a trip to memory).
+  if (blockIdx.x == 0) {
+    for (uint32_t g = threadIdx.x; g < w.G; g += kFusedThreads) {
+      if (dispatch_group_overflows(w, rows(), g)) atomicOr(w.faults, kFaultTooManyTokens);
+    }
   }
 }
 
@@ -393,19 +346,19 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab)
   __shared__ uint64_t s_scale[kWave];
   __shared__ int64_t s_step[kWave];
   const uint32_t v = blockIdx.x;
-  const uint32_t g = v / w.M;
+  const uint32_t g = group_of(w, v);
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
   if (t >= dispatch_group_tokens(w, tab, g)) return;
-  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  const DispatchRank &src = tab.at(sender_of(w, g, t));
   if (threadIdx.x < w.K) {
     uint64_t dst_row = 0, dst_scale = 0;
     int64_t step = 0;
     const uint32_t e = as_global(src.indices)[(size_t)t * w.K + threadIdx.x];
     const uint32_t slot = as_global(w.slot_map)[(size_t)v * w.K + threadIdx.x];
     if (e < w.E && slot != kInvalidSlot) {
-      const DispatchRank &dst = tab.at(e / w.L);
-      const uint32_t el = e % w.L;
+      const DispatchRank &dst = tab.at(owner_of(w, e));
+      const uint32_t el = local_of(w, e);
       if (slot < dst.x_rows) {
         dst_row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
                                              (int64_t)slot * dst.x_stride_row);
@@ -443,13 +396,15 @@ __global__ __launch_bounds__(256) void dispatch_scatter_long(WorldDev w, DT tab)
   }
 }
 
-// Number of waves a row's K copies are spread over: few tokens -> more waves,
-// so that the launch still covers the 256 CUs (the row re-reads hit L2).
-uint32_t fused_lds_bytes(const WorldDev &w, uint32_t tokens_per_block, bool inline_table) {
-  const uint32_t table = inline_table ? (uint32_t)sizeof(InlineDispatch) : 0u;
-  return table + tokens_per_block * w.K * 28u + (w.E + w.G) * (uint32_t)sizeof(uint32_t);
+// LDS of a dispatch_fused workgroup: the rank table (when it came inline), the histogram and
+// the mask of the workgroup's own tokens.
+uint32_t fused_lds_bytes(const WorldDev &w, bool inline_table) {
+  const uint32_t table = inline_table ? w.R * (uint32_t)sizeof(DispatchRank) : 0u;
+  return table + 2u * w.E * (uint32_t)sizeof(uint32_t);
 }
 
+// Number of waves a row's K copies are spread over: few tokens -> more waves,
+// so that the launch still covers the 256 CUs (the row re-reads hit L2).
 uint32_t pick_ksplit(const WorldDev &w, uint32_t max_split) {
   const uint64_t tokens = (uint64_t)w.G * w.M;
   uint32_t ksplit = 1;
@@ -513,7 +468,16 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, bool routed, hipStream_t 
   } while (0)
   if (routed) {
     PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter);
-  } else {
+  }
+#undef PPLX_LAUNCH_LARGE_ROW_VARIANT
+  // (rows beyond 16 KiB leave no registers for the slot arithmetic: slots_in_scatter() sends
+  // them through route_slots and the kernel above)
+#define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL)                                                    \
+  do {                                                                                           \
+    if (per_lane <= 16) PPLX_LAUNCH_ROW_VARIANT(KERNEL, 16, false);                              \
+    else return (int)hipErrorInvalidValue;                                                       \
+  } while (0)
+  if (!routed) {
     PPLX_DISPATCH_ROW_VARIANTS(dispatch_scatter_slots);
   }
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -538,7 +502,7 @@ int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipSt
   while (ksplit * 2 <= w.K && tokens_per_block * ksplit * 2 <= kWaves && (uint64_t)tokens * ksplit < 1024) ksplit *= 2;
   const uint32_t kper = (w.K + ksplit - 1) / ksplit;
   const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(kWaves * kWave);
-  const uint32_t lds = fused_lds_bytes(w, tokens_per_block, DT::kInline);
+  const uint32_t lds = fused_lds_bytes(w, DT::kInline && w.R <= kInlineRanks);
   // Rows that fit the last-level cache with room to spare are written through into it.
   const uint64_t row_bytes = (uint64_t)tokens * w.K * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
@@ -562,7 +526,7 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hi
   span.slot_out = w.slot_map;
   // Steps of several tiles leave the last routing launch out: the scatter's waves work their
   // own slots out of the tiles' tables.
-  const bool slots_in_scatter = w.num_tiles > 1 && scatter_has_register_rows(w);
+  const bool slots_in_scatter = w.num_tiles > 1 && (w.Hb / 16 + kWave - 1) / kWave <= 16;
   if (slots_in_scatter) {
     span.tile_mask = reinterpret_cast<unsigned long long *>(
         reinterpret_cast<uint8_t *>(w.tile_cnt) + route_tables(w.num_tiles, w.tile_chunks, w.E).mask_offset);
@@ -590,7 +554,7 @@ bool dispatch_is_fused(const WorldDev &w) {
   // 40 / 35; 4 KiB rows, top-8 of 64: 19 / 25, 26 / 32, 34 / 36, 49 / 49.  The one-launch form pays
   // while the routing launches (about 10 us of latency) weigh more than the scatter's better rate.
   const uint64_t tokens = (uint64_t)w.G * w.M;
-  return tokens <= kFusedMaxTokens && row_has_register_variant(w) && fused_lds_bytes(w, 16, true) <= 60 * 1024;
+  return tokens <= kFusedMaxTokens && row_has_register_variant(w) && fused_lds_bytes(w, true) <= 60 * 1024;
 }
 
 int launch_bind_dispatch(const WorldDev &w, const BindDispatchBatch &b, void *stream) {

@@ -44,10 +44,10 @@ __device__ __forceinline__ RouteToken route_token(const WorldDev &w, const DT &t
   RouteToken r;
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   r.v = span.v_begin + i;
-  r.g = r.v / w.M;
+  r.g = group_of(w, r.v);
   r.t = r.v - r.g * w.M;
   r.in_span = i < span.v_count && r.g < w.G;
-  const DispatchRank &src = tab.at(r.in_span ? r.g * w.dp + r.t % w.dp : 0);
+  const DispatchRank &src = tab.at(r.in_span ? sender_of(w, r.g, r.t) : 0);
   r.row_exists = r.in_span && r.t < src.m;
   r.n_group = r.in_span ? dispatch_group_tokens(w, tab, r.g) : 0;
   r.idx = as_global(src.indices) + (size_t)r.t * w.K;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(1024) void route_count(WorldDev w, DT tab, RouteSpa
 __device__ __forceinline__ uint32_t slots_from_masks(const WorldDev &w, uint32_t v, uint32_t lane, uint32_t e) {
   const uint32_t chunks = w.tile_chunks;
   const uint32_t chunk_abs = v / kWave;
-  const uint32_t tile = chunk_abs / chunks;
+  const uint32_t tile = chunk_abs >> __builtin_ctz(chunks);  // (a tile is a power of two of chunks)
   const uint32_t c = chunk_abs - tile * chunks;
   const unsigned long long below = (1ull << (v & (kWave - 1))) - 1ull;
   bool has_row = lane < w.K && e < w.E;
@@ -163,8 +163,8 @@ __global__ __launch_bounds__(256) void route_scan(WorldDev w, DT tab, RouteSpan 
     if (SPLIT) {
       span.counts_out[e] = carry;
     } else {
-      const DispatchRank &owner = tab.at(e / w.L);
-      as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)carry;
+      const DispatchRank &owner = tab.at(owner_of(w, e));
+      as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)carry;
     }
   }
 }
@@ -213,8 +213,8 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
       if (SPLIT) {
         span.counts_out[e] = running;
       } else {
-        const DispatchRank &owner = tab.at(e / w.L);
-        as_global(owner.out_num_tokens)[(int64_t)(e % w.L) * owner.out_num_tokens_stride] = (int32_t)running;
+        const DispatchRank &owner = tab.at(owner_of(w, e));
+        as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)running;
       }
     }
   }

@@ -50,8 +50,8 @@ __device__ __forceinline__ Destination resolve_destination(const WorldDev &w, co
                                                            uint32_t slot, bool report) {
   Destination d;
   if (e < w.E && slot != kInvalidSlot) {
-    const DispatchRank &dst = tab.at(e / w.L);
-    const uint32_t el = e % w.L;
+    const DispatchRank &dst = tab.at(owner_of(w, e));
+    const uint32_t el = local_of(w, e);
     if (slot < dst.x_rows) {
       d.row = reinterpret_cast<uint64_t>(dst.expert_x + (int64_t)el * dst.x_stride_expert +
                                          (int64_t)slot * dst.x_stride_row);

@@ -31,11 +31,11 @@ template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev sp, uint32_t write_through) {
   const uint32_t lane = lane_id();
   const uint32_t v = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
-  const uint32_t g = v / w.M;
+  const uint32_t g = group_of(w, v);
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
   if (t >= dispatch_group_tokens(w, tab, g)) return;
-  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  const DispatchRank &src = tab.at(sender_of(w, g, t));
   const uint32_t nvec = w.Hb / 16;
   const PPLX_GLOBAL u32x4 *row =
       as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
@@ -90,11 +90,11 @@ __global__ __launch_bounds__(256) void split_pack(WorldDev w, DT tab, SplitDev s
 template <class DT>
 __global__ __launch_bounds__(256) void split_pack_long(WorldDev w, DT tab, SplitDev sp) {
   const uint32_t v = blockIdx.x;
-  const uint32_t g = v / w.M;
+  const uint32_t g = group_of(w, v);
   const uint32_t t = v - g * w.M;
   if (g >= w.G) return;
   if (t >= dispatch_group_tokens(w, tab, g)) return;
-  const DispatchRank &src = tab.at(g * w.dp + t % w.dp);
+  const DispatchRank &src = tab.at(sender_of(w, g, t));
   const uint32_t nvec = w.Hb / 16;
   const PPLX_GLOBAL u32x4 *row =
       as_global(reinterpret_cast<const u32x4 *>(src.dp_x + (int64_t)t * src.dp_x_stride_row));
@@ -116,8 +116,8 @@ template <class DT>
 __device__ __forceinline__ void publish_counts(const WorldDev &w, const DT &tab, const SplitDev &sp) {
   if (blockIdx.x != 0) return;
   for (uint32_t e = threadIdx.x; e < w.E; e += blockDim.x) {
-    const DispatchRank &dst = tab.at(e / w.L);
-    as_global(dst.out_num_tokens)[(int64_t)(e % w.L) * dst.out_num_tokens_stride] = (int32_t)as_global(sp.gcnt)[e];
+    const DispatchRank &dst = tab.at(owner_of(w, e));
+    as_global(dst.out_num_tokens)[(int64_t)local_of(w, e) * dst.out_num_tokens_stride] = (int32_t)as_global(sp.gcnt)[e];
   }
 }
 
@@ -154,8 +154,8 @@ __global__ __launch_bounds__(256) void split_unpack(WorldDev w, DT tab, SplitDev
   for (int v = 0; v < NV; ++v) settle(x[v]);
   settle(sc);
   if (e >= w.E || slot == kInvalidSlot) return;
-  const DispatchRank &dst = tab.at(e / w.L);
-  const uint32_t el = e % w.L;
+  const DispatchRank &dst = tab.at(owner_of(w, e));
+  const uint32_t el = local_of(w, e);
   if (slot >= dst.x_rows) {
     if (lane == 0) atomicOr(w.faults, kFaultRowDropped);
     return;
@@ -190,8 +190,8 @@ __global__ __launch_bounds__(256) void split_unpack_long(WorldDev w, DT tab, Spl
   const uint32_t e = as_global(sp.gexp)[pair];
   const uint32_t slot = as_global(w.slot_map)[pair];
   if (e >= w.E || slot == kInvalidSlot) return;
-  const DispatchRank &dst = tab.at(e / w.L);
-  const uint32_t el = e % w.L;
+  const DispatchRank &dst = tab.at(owner_of(w, e));
+  const uint32_t el = local_of(w, e);
   if (slot >= dst.x_rows) {
     if (threadIdx.x == 0) atomicOr(w.faults, kFaultRowDropped);
     return;
@@ -215,8 +215,8 @@ __global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, Sp
   const uint32_t lane = lane_id();
   const uint64_t pair = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
   if (pair >= (uint64_t)w.G * w.M * w.K) return;
-  const uint32_t v = (uint32_t)(pair / w.K);
-  const uint32_t g = v / w.M;
+  const uint32_t v = fast_div((uint32_t)pair, w.by_K);
+  const uint32_t g = group_of(w, v);
   const uint32_t t = v - g * w.M;
   const CombineRank &head = tab.at(g * w.dp);
   if (t >= combine_rank_tokens(w, head)) return;
@@ -227,13 +227,13 @@ __global__ __launch_bounds__(256) void split_combine_send(WorldDev w, CT tab, Sp
   const uint32_t e = as_global(head.indices)[pair - (uint64_t)g * w.M * w.K];
   const uint32_t slot = as_global(w.slot_map)[pair];
   if (e >= w.E || slot == kInvalidSlot) return;
-  const CombineRank &own = tab.at(e / w.L);
+  const CombineRank &own = tab.at(owner_of(w, e));
   if (slot >= own.y_rows) {
     if (lane == 0) atomicOr(w.faults, kFaultBadSlot);
     return;
   }
   const uint8_t *src = reinterpret_cast<const uint8_t *>(own.expert_y) +
-                       ((int64_t)(e % w.L) * own.y_stride_expert + (int64_t)slot * own.y_stride_row) * elem_bytes;
+                       ((int64_t)local_of(w, e) * own.y_stride_expert + (int64_t)slot * own.y_stride_row) * elem_bytes;
   const PPLX_GLOBAL u32x4 *row = as_global(reinterpret_cast<const u32x4 *>(src));
   PPLX_GLOBAL u32x4 *out = as_global(reinterpret_cast<u32x4 *>(sp.stage_y + pair * sp.y_row_bytes));
   const uint32_t nvec = (uint32_t)(sp.y_row_bytes / 16);

@@ -11,6 +11,7 @@
 #include <cmath>
 #include <string>
 
+#include "a2a_device.h"
 #include "harness.h"
 
 using namespace harness;
@@ -160,6 +161,27 @@ bool run_case(const Geometry &geo, Mode mode, hipStream_t stream) {
     for (uint32_t r = 0; r < geo.R; ++r) all.push_back(dispatch_args(r));
     A2A_OK(pplx_a2a_world_dispatch(world, all.data(), stream));
   } else if (mode == PER_RANK) {
+    // A step that stops half way (all ranks but the last have called) is given up: the world is
+    // idle again, nothing ran, and the whole step is made from the first rank on.
+    {
+      uint32_t recorded = 0, dropped = 0;
+      for (uint32_t r = 0; r + 1 < geo.R; ++r) {
+        auto a = dispatch_args(r);
+        A2A_OK(pplx_a2a_dispatch(ranks[r], &a, PPLX_A2A_SPLIT_NONE, stream));
+      }
+      A2A_OK(pplx_a2a_world_recorded_calls(world, 0, PPLX_A2A_SPLIT_NONE, &recorded));
+      auto again = dispatch_args(0);
+      const int twice = pplx_a2a_dispatch(ranks[0], &again, PPLX_A2A_SPLIT_NONE, stream);
+      A2A_OK(pplx_a2a_world_abandon_step(world, PPLX_A2A_ABANDON_DISPATCH | PPLX_A2A_ABANDON_COMBINE, &dropped));
+      uint32_t after = ~0u;
+      A2A_OK(pplx_a2a_world_recorded_calls(world, 0, PPLX_A2A_SPLIT_NONE, &after));
+      if (recorded != geo.R - 1 || twice != PPLX_A2A_INVALID_STATE || dropped != geo.R - 1 || after != 0 ||
+          pplx_a2a_world_abandon_step(world, 0, nullptr) != PPLX_A2A_INVALID_ARGUMENT) {
+        printf("  FAIL %s [%s]: abandon: recorded %u, second call %d, dropped %u, left %u\n", geo.name,
+               mode_name(mode), recorded, twice, dropped, after);
+        return false;
+      }
+    }
     for (uint32_t r = 0; r < geo.R; ++r) {
       auto a = dispatch_args(r);
       A2A_OK(pplx_a2a_dispatch(ranks[r], &a, PPLX_A2A_SPLIT_NONE, stream));
@@ -277,9 +299,48 @@ bool run_case(const Geometry &geo, Mode mode, hipStream_t stream) {
   return ok;
 }
 
+// The division helper of the kernels (a2a_device.h) against the hardware's own, on the host:
+// every divisor a geometry can produce in the small range, large ones in strides, numerators
+// around every multiple's edge and across the 32-bit range.
+bool check_fast_div() {
+  uint64_t checked = 0;
+  auto check = [&](uint32_t n, uint32_t d, const pplx_amd::FastDiv &f) {
+    ++checked;
+    if (pplx_amd::fast_div(n, f) == n / d) return true;
+    printf("  FAIL fast_div(%u, %u) = %u, expected %u\n", n, d, pplx_amd::fast_div(n, f), n / d);
+    return false;
+  };
+  std::vector<uint32_t> divisors;
+  for (uint32_t d = 1; d <= 8200; ++d) divisors.push_back(d);
+  for (uint64_t d = 8209; d < (1ull << 32); d = d * 3 / 2 + 7) divisors.push_back((uint32_t)d);
+  for (uint32_t d : {0x3fffffffu, 0x40000000u, 0x40000001u, 0x7fffffffu, 0x80000000u, 0x80000001u, 0xfffffffeu, 0xffffffffu})
+    divisors.push_back(d);
+  for (uint32_t d : divisors) {
+    const pplx_amd::FastDiv f = pplx_amd::make_fast_div(d);
+    for (uint32_t n = 0; n < 300; ++n)
+      if (!check(n, d, f)) return false;
+    for (uint64_t q = 1; q * d < (1ull << 32) && q < 40; ++q)
+      for (int64_t delta = -2; delta <= 2; ++delta) {
+        const int64_t n = (int64_t)(q * d) + delta;
+        if (n >= 0 && n < (1ll << 32) && !check((uint32_t)n, d, f)) return false;
+      }
+    uint32_t x = d * 2654435761u + 12345u;
+    for (int i = 0; i < 200; ++i) {
+      x = x * 1664525u + 1013904223u;
+      if (!check(x, d, f) || !check(x >> (i % 31), d, f)) return false;
+    }
+    for (uint32_t n : {0xffffffffu, 0xfffffffeu, 0x80000000u, 0x7fffffffu})
+      if (!check(n, d, f)) return false;
+  }
+  printf("  pass [fast_div: %llu quotients against the hardware's]\n", (unsigned long long)checked);
+  return true;
+}
+
 }  // namespace
 
-int main() {
+int main(int argc, char **argv) {
+  if (!check_fast_div()) return 1;
+  if (argc > 1 && std::string(argv[1]) == "--host-only") return 0;
   int n_dev = 0;
   if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
     fprintf(stderr, "test_a2a: no GPU visible\n");

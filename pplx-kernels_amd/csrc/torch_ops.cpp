@@ -284,6 +284,9 @@ void dispatch_core(fptr_t ptr, const at::Tensor &outExpertNumTokens, const at::T
                    const at::Tensor &indices, const at::Tensor *boundM, bool doSend, bool doRecv) {
   std::lock_guard<std::mutex> lock(g_mu);
   World *world = nullptr;
+  // What a failure means: refused arguments give the step being assembled up (below); call-order
+  // and runtime errors leave the recorded calls alone.
+  bool arguments_refused = true;
   try {
     // (a handle that is unknown is reported after the tensor checks, which need no handle)
     auto found = g_ranks.find(ptr);
@@ -338,23 +341,17 @@ void dispatch_core(fptr_t ptr, const at::Tensor &outExpertNumTokens, const at::T
 
     // Split calls go through staging that dispatch / combine never allocate; the reference's
     // callers do not know of it, so it is reserved the first time a rank splits a call.
+    arguments_refused = false;
     if (mode != PPLX_A2A_SPLIT_NONE) reserve_split_locked(*world, 0);
     // The library selects the world's device for the launch and restores the caller's; the
     // stream is the current one of the tensors' device (csrc/bindings/all_to_all_ops.cpp:163,194).
     const int st = pplx_a2a_dispatch((pplx_a2a_t *)ptr, &a, mode, current_stream_of(indices));
     settle_held(*world, ref.rank, 0, mode, st == PPLX_A2A_OK,
                 {&outExpertNumTokens, &outExpertX, outExpertXScale, &dpX, dpXScale, &indices, boundM});
-    if (st == PPLX_A2A_INVALID_ARGUMENT) {
-      // (thrown from here so that the handler below sees an argument error, not a state error)
-      TORCH_CHECK(false, "pplx_kernels: ", status_name(st), ": ", pplx_a2a_last_error());
-    }
-    if (st != PPLX_A2A_OK) {
-      const std::string msg = std::string("pplx_kernels: ") + status_name(st) + ": " + pplx_a2a_last_error();
-      world = nullptr;  // call-order and runtime errors leave the recorded calls alone
-      TORCH_CHECK(false, msg);
-    }
+    arguments_refused = st == PPLX_A2A_INVALID_ARGUMENT;
+    A2A_CHECK(st);
   } catch (const c10::Error &err) {
-    const uint32_t dropped = abandon_assembly(world, 0);
+    const uint32_t dropped = arguments_refused ? abandon_assembly(world, 0) : 0;
     if (dropped == 0) throw;
     A2A_RETHROW_ABANDONED(err, "dispatch", dropped);
   }
@@ -365,6 +362,7 @@ void combine_core(fptr_t ptr, const at::Tensor &outTokens, const at::Tensor &ind
                   const at::Tensor &expertY, const at::Tensor *boundM, bool doSend, bool doRecv) {
   std::lock_guard<std::mutex> lock(g_mu);
   World *world = nullptr;
+  bool arguments_refused = true;
   try {
     auto found = g_ranks.find(ptr);
     if (found != g_ranks.end()) world = found->second.world;
@@ -397,19 +395,14 @@ void combine_core(fptr_t ptr, const at::Tensor &outTokens, const at::Tensor &ind
     a.m = (uint32_t)indices.size(0);
     a.bound_m = boundM ? static_cast<const uint32_t *>(boundM->data_ptr()) : nullptr;
 
+    arguments_refused = false;
     if (mode != PPLX_A2A_SPLIT_NONE) reserve_split_locked(*world, (int)expertY.element_size());
     const int st = pplx_a2a_combine((pplx_a2a_t *)ptr, &a, mode, current_stream_of(indices));
     settle_held(*world, ref.rank, 1, mode, st == PPLX_A2A_OK, {&outTokens, &indices, &weights, &expertY, boundM});
-    if (st == PPLX_A2A_INVALID_ARGUMENT) {
-      TORCH_CHECK(false, "pplx_kernels: ", status_name(st), ": ", pplx_a2a_last_error());
-    }
-    if (st != PPLX_A2A_OK) {
-      const std::string msg = std::string("pplx_kernels: ") + status_name(st) + ": " + pplx_a2a_last_error();
-      world = nullptr;
-      TORCH_CHECK(false, msg);
-    }
+    arguments_refused = st == PPLX_A2A_INVALID_ARGUMENT;
+    A2A_CHECK(st);
   } catch (const c10::Error &err) {
-    const uint32_t dropped = abandon_assembly(world, 1);
+    const uint32_t dropped = arguments_refused ? abandon_assembly(world, 1) : 0;
     if (dropped == 0) throw;
     A2A_RETHROW_ABANDONED(err, "combine", dropped);
   }

@@ -149,6 +149,39 @@ def test_binding_checks_fire_before_the_device():
     assert (ops.split_mode(True, True), ops.split_mode(True, False), ops.split_mode(False, True)) == (0, 1, 2)
 
 
+def test_operator_layer_checks_fire_before_the_device():
+    """The same checks in the compiled operator layer (pplx_kernels._C), which the per-rank
+    API goes through: CPU tensors are refused with the reference's messages, wrong Python types
+    are TypeErrors, and a CPU tensor handed to the registered op finds no kernel."""
+    C = ops._C
+    n, k, h = 4, 2, 64
+    i32 = torch.zeros(2, dtype=torch.int32)
+    x3 = torch.zeros(2, 8, h, dtype=torch.bfloat16)
+    x2 = torch.zeros(n, h, dtype=torch.bfloat16)
+    idx = torch.zeros(n, k, dtype=torch.uint32)
+    with pytest.raises(RuntimeError, match="Tensor outExpertNumTokens must be on GPU"):
+        C.dispatch(0, i32, x3, None, x2, None, idx, None, True, True)
+    with pytest.raises(RuntimeError, match="Tensor outTokens must be on GPU"):
+        C.combine(0, x2, idx, torch.zeros(n, k), x3, None, True, True)
+    with pytest.raises(TypeError, match="dp_x must be a Tensor, not NoneType"):
+        C.dispatch(0, i32, x3, None, None, None, idx, None, True, True)
+    with pytest.raises(TypeError, match="takes 10 positional arguments but 3 were given"):
+        C.dispatch(0, i32, x3)
+    with pytest.raises(TypeError, match="fptr must be an int"):
+        C.combine("0", x2, idx, torch.zeros(n, k), x3, None, True, True)
+    with pytest.raises(NotImplementedError):
+        torch.ops.pplx_kernels.all_to_all_intranode_dispatch(0, i32, x3, None, x2, None, idx, None, True, True)
+    with pytest.raises(RuntimeError, match="unknown all-to-all handle"):
+        torch.ops.pplx_kernels.all_to_all_destroy(12345)
+    with pytest.raises(RuntimeError, match="the handle has been destroyed"):
+        C.world_ptr(12345)
+    assert C.is_live(12345) is False
+    with pytest.raises(RuntimeError, match="negative rank"):
+        torch.ops.pplx_kernels.all_to_all_intranode_create(8, 8, 2, -1, 4, 1, 64, 128, 0, "g")
+    with pytest.raises(RuntimeError, match="negative or zero size"):
+        torch.ops.pplx_kernels.all_to_all_internode_create(8, 8, 2, 0, 0, 1, 64, 128, 0)
+
+
 def test_op_schemas_match_the_reference():
     """csrc/bindings/all_to_all_ops.cpp:329-391: names, mutability and argument order."""
     for transport in ("intranode", "internode"):

@@ -405,6 +405,15 @@ def test_first_split_step_is_capturable_once_reserved():
         expected = check_dispatch_against_oracle(step)
         check_combine_against_oracle(step, expected.slot_map)
     ops.check_status(lib.pplx_a2a_graph_destroy(graph))
+    # The graph holds the address of the 2-byte combine staging: widening it (which would free
+    # it) is refused from now on, through the C ABI and through an f32 split combine alike.
+    assert lib.pplx_a2a_world_reserve_split(world.ptr, 4) == 2
+    assert b"captured into a graph" in lib.pplx_a2a_last_error()
+    assert lib.pplx_a2a_world_reserve_split(world.ptr, 2) == 0
+    with pytest.raises(RuntimeError, match="captured into a graph"):
+        ranks[0].combine(
+            **{**_combine_kw(step, 0), "expert_y": step.expert_y[0].float()}, do_send=True, do_recv=False
+        )
     for a in ranks:
         a.destroy()
 

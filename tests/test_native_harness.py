@@ -18,10 +18,18 @@ def test_cpp_harness_passes():
     print(proc.stdout[-4000:], proc.stderr[-4000:])
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert "ALL PASSED" in proc.stdout
-    assert proc.stdout.count("  pass [") == 18
+    assert proc.stdout.count("  pass [") == 19  # 6 geometries x 3 call forms + the division helper
 
 
 def test_cpp_harness_is_built_and_linked_against_the_library():
     assert os.path.exists(BIN)
     out = subprocess.run(["ldd", BIN], capture_output=True, text=True).stdout
     assert "libpplx_kernels.so" in out and "not found" not in out.split("libpplx_kernels.so")[1].splitlines()[0]
+
+
+def test_division_helper_of_the_kernels_matches_integer_division():
+    """The kernels divide by launch constants (tokens per group, experts per rank ...) with a
+    multiply-high and two shifts; the host part of the C++ harness compares that helper with
+    the hardware's division on millions of (numerator, divisor) pairs.  Needs no GPU."""
+    proc = subprocess.run([BIN, "--host-only"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0 and "pass [fast_div" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-2000:]

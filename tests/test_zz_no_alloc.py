@@ -10,7 +10,16 @@ import ctypes
 import pytest
 import torch
 
-from tests.all_to_all_utils import FP8, DeviceStep, WorkloadSpec, expert_counts, generate, make_world
+from tests.all_to_all_utils import (
+    FP8,
+    DeviceStep,
+    WorkloadSpec,
+    check_combine_against_oracle,
+    check_dispatch_against_oracle,
+    expert_counts,
+    generate,
+    make_world,
+)
 
 pytestmark = pytest.mark.gpu
 
@@ -105,6 +114,9 @@ def _compare(spec, groups, fault_word, cap=None, one_call=False):
         assert not torch.isnan(b.float()).any()
         assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"combine differs on rank {r}"
         assert torch.isnan(got.out_tokens[r][n:].float()).all()
+    # ... and, like the world path, equal to the CPU oracle
+    expected = check_dispatch_against_oracle(got)
+    check_combine_against_oracle(got, expected.slot_map, use_numpy=True)
 
 
 def test_static_step_matches_the_world_path_on_calls_in_a_row():
@@ -215,3 +227,55 @@ def test_static_step_replays_from_a_graph():
     ops.check_status(lib.pplx_a2a_graph_destroy(graph))
     assert world.faults() == 0
     world.destroy()
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import ctypes, sys
+import torch
+sys.path[:0] = [{pkg!r}, {root!r}]
+from pplx_kernels import ops
+from tests.all_to_all_utils import DeviceStep, WorkloadSpec, generate
+from tests.test_zz_no_alloc import _config, _pack, _spec
+
+lib = ops.load_library()
+spec = _spec(name="first", world_size=4, num_experts=16, experts_per_token=4, hidden_dim=256,
+             max_num_tokens=24, in_dtype=torch.bfloat16)
+step = DeviceStep(spec, generate(spec))
+cfg = _config(ops, spec)
+d_args, c_args = _pack(ops, spec, step)
+stream = torch.cuda.Stream()
+torch.cuda.synchronize()
+graph = ctypes.c_void_p()
+with torch.cuda.stream(stream):
+    ops.check_status(lib.pplx_a2a_graph_begin_capture(stream.cuda_stream))
+    st = lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, d_args, c_args, None, stream.cuda_stream)
+    msg = lib.pplx_a2a_last_error().decode()
+    ops.check_status(lib.pplx_a2a_graph_end_capture(stream.cuda_stream, ctypes.byref(graph)))
+    ops.check_status(lib.pplx_a2a_graph_destroy(graph))
+    assert st == 2 and "cannot be captured" in msg, (st, msg)
+    ops.check_status(lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, d_args, c_args, None, stream.cuda_stream))
+    stream.synchronize()
+    ops.check_status(lib.pplx_a2a_graph_begin_capture(stream.cuda_stream))
+    st = lib.pplx_a2a_static_step(ctypes.byref(cfg), 0, d_args, c_args, None, stream.cuda_stream)
+    ops.check_status(lib.pplx_a2a_graph_end_capture(stream.cuda_stream, ctypes.byref(graph)))
+    assert st == 0, lib.pplx_a2a_last_error()
+    ops.check_status(lib.pplx_a2a_graph_launch(graph, stream.cuda_stream))
+    stream.synchronize()
+    ops.check_status(lib.pplx_a2a_graph_destroy(graph))
+print("first-call-ok")
+"""
+
+
+def test_first_static_step_of_a_process_cannot_be_captured():
+    """The first call on a device sets the library up (address of the scratch array, the
+    device's LDS size): under stream capture it is refused with a status code, and works once
+    one eager call has been made.  Needs a process in which nothing has touched the library
+    yet, hence the child process."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = _FIRST_CALL_UNDER_CAPTURE.format(pkg=os.path.join(root, "pplx-kernels_amd"), root=root)
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0 and "first-call-ok" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-3000:]
