@@ -8,16 +8,26 @@ steps rotate over several independent buffer sets, so every timed step touches m
 last used several steps ago.
 
 Prints ONE JSON line.  ``value`` is the mean step latency in microseconds on the workload the
-metric is quoted on (C2: DeepSeek-V3 shape, 128 tokens/rank, 8 simulated ranks).  How a step is
-launched is fixed by rule, not picked per run: eager launches of a step whose arguments were
-checked and packed once (``LoopbackWorld.bind``: two library calls per step) for every workload
-but the decode shape C3, which is ONE captured hipGraph replayed 1000 times; the other form is
-reported next to it.  ``workloads`` holds a compact entry for each of C1..C5.
+metric is quoted on (C2: DeepSeek-V3 shape, 128 tokens/rank, 8 simulated ranks), over exactly
+``--steps`` steps in one timed region.  Every workload C1..C5 is measured in the same three
+launch forms under fixed keys, on the same rotating buffer sets:
+
+* ``bound_eager_step_us`` (= ``step_us``): eager launches of a step whose arguments were checked
+  and packed once (``LoopbackWorld.bind``: two library calls per step);
+* ``graph_step_us``: the same step captured into one hipGraph per buffer set and replayed;
+* ``per_rank_api_step_us``: the reference's own call path, ``AllToAll.dispatch`` once per
+  simulated rank and then ``AllToAll.combine`` once per rank, eagerly, arguments checked on
+  every call (what ``tests/bench_all_to_all.py`` of the reference times per rank).
+
+The decode shape C3 additionally carries ``graph_replay_1000x_us``: ONE captured graph over ONE
+buffer set replayed 1000 times, the form its specification names; 12.5 MB replayed back to back
+stay in the last-level cache, so that figure is cache-resident and carries no HBM fraction.
 ``roofline`` is for the dominant kernel of the headline workload (``combine_gather``):
 algorithmic bytes per launch divided by its mean duration, measured with HIP events around graph
 replays that contain only launches of that kernel; ``traffic`` is read from the rocprofv3 counter
-summary under ``profiles/``.  ``cpu_baseline`` times the oracle's vectorised torch CPU port of the
-same step on this host's cores.
+summary under ``profiles/`` when that summary was made with the library that is running.  Every
+workload carries a ``cpu_baseline``: the oracle's vectorised torch CPU port of the same step on
+the same inputs, on this host's cores.
 """
 
 from __future__ import annotations
@@ -42,19 +52,31 @@ LLC_BYTES = 256 << 20
 GRAPH_REPLAYS_C3 = 1000
 
 
-def measured_traffic_bytes(workload: str, kernel: str):
-    """HBM bytes per launch of `kernel` from profiles/hbm_traffic_<workload>.txt (rocprofv3 --pmc
-    FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size in the same run); None when the
-    summary is not there.  Counters cannot be read from inside this script."""
+def measured_traffic_bytes(workload: str, kernel: str, build_id: str):
+    """(HBM bytes per launch of `kernel`, note) from profiles/hbm_traffic_<workload>.txt (rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size in the same run).  The summary
+    names the library it was measured with; bytes are None when it is missing or was made with
+    another build.  Counters cannot be read from inside this script."""
     path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}.txt")
     try:
-        for line in open(path):
-            fields = line.split()
-            if fields and fields[0] == kernel and re.fullmatch(r"[0-9.]+", fields[-1]):
-                return float(fields[-1]) * 1e6  # last column: total MB
+        lines = open(path).read().splitlines()
     except OSError:
-        pass
-    return None
+        return None, f"no counter summary {os.path.relpath(path, ROOT)}"
+    measured_with = None
+    for line in lines:
+        m = re.search(r"library build id:\s*([0-9a-f]+)", line)
+        if m:
+            measured_with = m.group(1)
+    if measured_with != build_id:
+        return None, (
+            f"{os.path.relpath(path, ROOT)} was measured with library build {measured_with}, "
+            f"this run uses {build_id}: counters not carried over"
+        )
+    for line in lines:
+        fields = line.split()
+        if fields and fields[0] == kernel and re.fullmatch(r"[0-9.]+", fields[-1]):
+            return float(fields[-1]) * 1e6, f"{os.path.relpath(path, ROOT)} (library build {build_id})"
+    return None, f"{os.path.relpath(path, ROOT)} has no line for {kernel}"
 
 
 def build_steps(spec, groups, cap, n_sets):
@@ -92,17 +114,10 @@ def time_graphs(graphs, order, stream, warmup, repeats=1):
     return start.elapsed_time(end) * 1e3 / (len(order) * repeats)
 
 
-def time_bound(bound, order, stream, warmup, dispatch=True, combine=True):
-    """Mean microseconds per step (or per phase) of eager launches of bound steps, HIP events on
-    the launch stream."""
+def time_steps(run, order, stream, warmup):
+    """Mean microseconds per call of run(i) over `order` (buffer-set indices) in ONE timed region,
+    HIP events on the launch stream, which is also the current stream inside run."""
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-
-    def run(i):
-        if dispatch:
-            bound[i].dispatch(stream)
-        if combine:
-            bound[i].combine(stream)
-
     with torch.cuda.stream(stream):
         for i in range(warmup):
             run(order[i % len(order)])
@@ -122,6 +137,9 @@ def capture(world, stream, body):
         with world.capture() as cap:
             body()
     return cap.graph
+
+
+EXTRA_REGIONS = 4  # further timed regions of the same length, for the spread
 
 
 def measure_workload(name, spec, steps_k, warmup):
@@ -145,58 +163,79 @@ def measure_workload(name, spec, steps_k, warmup):
     torch.cuda.synchronize()
     order = [i % n_sets for i in range(steps_k)]
 
-    # Eager launches of steps packed once (LoopbackWorld.bind): two library calls per step.
+    # 1. eager launches of steps packed once (LoopbackWorld.bind): two library calls per step
     bound = [st.bind_world(world) for st in steps]
-    bound_us = time_bound(bound, order, stream, warmup)
-    d_us = time_bound(bound, order, stream, warmup, combine=False)
-    c_us = time_bound(bound, order, stream, warmup, dispatch=False)
+    bound_us = time_steps(lambda i: (bound[i].dispatch(stream), bound[i].combine(stream)), order, stream, warmup)
+    more = [
+        time_steps(lambda i: (bound[i].dispatch(stream), bound[i].combine(stream)), order, stream, 0)
+        for _ in range(EXTRA_REGIONS)
+    ]
+    d_us = time_steps(lambda i: bound[i].dispatch(stream), order, stream, warmup)
+    c_us = time_steps(lambda i: bound[i].combine(stream), order, stream, warmup)
 
-    # The same step as a captured hipGraph.
+    # 2. the reference's call path: one AllToAll.dispatch per simulated rank, then one
+    # AllToAll.combine per rank (src/pplx_kernels/all_to_all.py:27-81), eagerly, on the same sets
+    ranks = world.ranks
+    per_rank_us = time_steps(
+        lambda i: (steps[i].dispatch_per_rank(ranks), steps[i].combine_per_rank(ranks)), order, stream, warmup
+    )
+
+    # 3. the same step as a captured hipGraph, one per buffer set
     def both(st):
         return lambda: (st.dispatch_world(world), st.combine_world(world))
 
+    graphs = [capture(world, stream, both(st)) for st in steps]
+    graph_us = time_graphs(graphs, order, stream, warmup)
+    replay_1000 = None
     if name == "C3":
-        # the decode shape: ONE graph, replayed 1000 times back to back
-        graph = capture(world, stream, both(steps[0]))
-        graph_us = time_graphs([graph], [0], stream, warmup, GRAPH_REPLAYS_C3)
-        graph.destroy()
-        graph_note = f"one hipGraph replayed {GRAPH_REPLAYS_C3} times"
-    else:
-        graphs = [capture(world, stream, both(st)) for st in steps]
-        graph_us = time_graphs(graphs, order, stream, warmup)
-        for g in graphs:
-            g.destroy()
-        graph_note = f"{n_sets} hipGraphs (one per buffer set), {len(order)} replays"
+        # the form the decode shape is specified in: ONE graph, replayed 1000 times back to back
+        replay_1000 = time_graphs([graphs[0]], [0], stream, warmup, GRAPH_REPLAYS_C3)
+    for g in graphs:
+        g.destroy()
     del bound
 
-    launch_form = "graph_replay" if name == "C3" else "bound_eager"
-    step_us = graph_us if name == "C3" else bound_us
     pairs = int(sum(g.n for g in groups) * spec.experts_per_token)
+    spread = [bound_us] + more
     out = {
         "workload": spec.name,
         "tokens": int(sum(g.n for g in groups)),
         "pairs": pairs,
         "rows_per_expert_capacity": cap,
         "buffer_sets": n_sets,
-        "steps_timed": len(order) if name != "C3" else GRAPH_REPLAYS_C3,
-        "launch_form": launch_form,
-        "step_us": step_us,
+        "steps_timed": len(order),
+        "launch_form": "bound_eager",
+        "step_us": bound_us,
+        "step_us_regions": {
+            "n": len(spread),
+            "mean": statistics.mean(spread),
+            "std": statistics.pstdev(spread),
+            "min": min(spread),
+            "note": f"{len(spread)} timed regions of {len(order)} steps each; step_us is the first",
+        },
         "bound_eager_step_us": bound_us,
         "graph_step_us": graph_us,
-        "graph_form": graph_note,
+        "per_rank_api_step_us": per_rank_us,
+        "per_rank_api_calls_per_step": 2 * spec.world_size,
         "dispatch_us": d_us,
         "combine_us": c_us,
         "dispatch_bytes": disp_b,
         "combine_bytes": comb_b,
-        "step_hbm_frac": (disp_b + comb_b) / step_us / 1e3 / HBM_PEAK_GBPS,
+        "step_hbm_frac": (disp_b + comb_b) / bound_us / 1e3 / HBM_PEAK_GBPS,
         "dispatch_hbm_frac": disp_b / d_us / 1e3 / HBM_PEAK_GBPS,
         "combine_hbm_frac": comb_b / c_us / 1e3 / HBM_PEAK_GBPS,
-        "step_GBps": (disp_b + comb_b) / step_us / 1e3,
+        "step_GBps": (disp_b + comb_b) / bound_us / 1e3,
         # the reference bench's one-way payload figures (tests/bench_all_to_all.py:131-139):
         # pairs x bytes per dispatched token, pairs x bytes per combined row
         "dispatch_payload_GBps": pairs * (spec.hidden_dim_bytes + spec.hidden_dim_scale_bytes) / d_us / 1e3,
         "combine_payload_GBps": pairs * spec.hidden_dim * spec.out_dtype.itemsize / c_us / 1e3,
     }
+    if replay_1000 is not None:
+        out["graph_replay_1000x_us"] = replay_1000
+        out["graph_replay_1000x_note"] = (
+            f"one hipGraph over one buffer set replayed {GRAPH_REPLAYS_C3} times back to back: the "
+            f"{(disp_b + comb_b) / 1e6:.1f} MB of a step stay in the 256 MB last-level cache, so this is a "
+            "cache-resident latency and no HBM fraction is derived from it"
+        )
     assert world.faults() == 0, "device-side fault bits set during the benchmark"
     world.destroy()
     return out, groups, steps
@@ -231,6 +270,11 @@ def combine_kernel_roofline(name, spec, steps, comb_b, steps_k):
     for g in k_graphs:
         g.destroy()
     world.destroy()
+    from pplx_kernels import ops
+
+    traffic, traffic_source = measured_traffic_bytes(
+        name, "combine_gather", ops.load_library().pplx_a2a_build_id().decode()
+    )
     return {
         "kernel": "combine_gather<bf16,bf16>",
         "bound": "hbm",
@@ -238,32 +282,38 @@ def combine_kernel_roofline(name, spec, steps, comb_b, steps_k):
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": comb_b / kernel_us / 1e3 / HBM_PEAK_GBPS,
-        "traffic": measured_traffic_bytes(name, "combine_gather"),
+        "traffic": traffic,
+        "traffic_source": traffic_source,
         "bytes_per_launch": comb_b,
         "avg_launch_us": kernel_us,
         "launches_timed": reps * n_sets * launches_per_graph,
     }
 
 
-def cpu_baseline(spec, groups, budget_s=20.0):
-    """The oracle's vectorised torch CPU port of one full step, on all host cores."""
+def cpu_baseline(spec, groups, budget_s=12.0):
+    """The oracle's vectorised torch CPU port of one full step (stable argsort on the expert id,
+    index_select / index_copy_ for dispatch; index_select + fp32 weighted sum for combine; it
+    restates the routing of the reference's tests/test_all_to_all.py:113-120,277-286), on all host
+    cores, on the inputs the GPU leg ran.  expert_y holds as many rows per expert as the busiest
+    expert receives, so that the 8192-token prefill fits host memory."""
     from oracle import a2a_oracle as orc
+    from pplx_kernels.workloads import expert_counts
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     M, E, K, H = spec.max_num_tokens, spec.num_experts, spec.experts_per_token, spec.hidden_dim
-    cap = M * spec.num_dp_groups
+    cap = max(int(expert_counts(groups, E).max()), 1)
     groups_t = [(g.x, g.x_scale, g.indices.to(torch.int64), g.n) for g in groups]
     weights_t = [g.weights for g in groups]
     # N(0,1) rows; one [cap, H] slab replicated per expert keeps the set-up short
-    slab = torch.randn(cap, H, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    slab = torch.randn(cap, H, generator=torch.Generator().manual_seed(1)).to(spec.expert_y_dtype)
     expert_y = slab.unsqueeze(0).expand(E, cap, H).contiguous()
     times = []
     t_all = time.perf_counter()
-    while len(times) < 5 or (time.perf_counter() - t_all < budget_s / 2 and len(times) < 15):
+    while len(times) < 3 or (time.perf_counter() - t_all < budget_s / 2 and len(times) < 15):
         t0 = time.perf_counter()
         _, _, _, slot_flat = orc.torch_dispatch(groups_t, M, E, K, cap)
-        orc.torch_combine(groups_t, weights_t, slot_flat, expert_y, torch.bfloat16)
+        orc.torch_combine(groups_t, weights_t, slot_flat, expert_y, spec.out_dtype)
         times.append(time.perf_counter() - t0)
         if time.perf_counter() - t_all > budget_s:
             break
@@ -272,8 +322,9 @@ def cpu_baseline(spec, groups, budget_s=20.0):
         "unit": "us",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{len(times)} full steps of the same workload (all {sum(g.n for g in groups)} tokens), "
-        "median; torch CPU stable-argsort scatter + fp32 gather-sum (oracle.a2a_oracle.torch_*)",
+        "sample": f"{len(times)} full steps of the same workload (all {sum(g.n for g in groups)} tokens, "
+        f"{cap} rows per expert), median; torch CPU stable-argsort scatter + fp32 gather-sum "
+        "(oracle.a2a_oracle.torch_*)",
     }
 
 
@@ -329,7 +380,10 @@ def counter_probe(spec, launches=3):
         step.combine_world(world)
         torch.cuda.synchronize()
     d, c = step.algorithmic_bytes()
-    print(json.dumps({"probe": spec.name, "dispatch_bytes": d, "combine_bytes": c, "copy_bytes_each_way": 1 << 30}))
+    from pplx_kernels import ops
+
+    print(json.dumps({"probe": spec.name, "dispatch_bytes": d, "combine_bytes": c, "copy_bytes_each_way": 1 << 30,
+                      "library_build_id": ops.load_library().pplx_a2a_build_id().decode()}))  # fmt: skip
     world.destroy()
 
 
@@ -343,9 +397,15 @@ def steps_for(name, steps_k):
 
 
 COMPACT_FIELDS = (
-    "workload", "tokens", "pairs", "buffer_sets", "steps_timed", "launch_form", "step_us", "bound_eager_step_us",
-    "graph_step_us", "dispatch_us", "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac",
+    "workload", "tokens", "pairs", "buffer_sets", "steps_timed", "launch_form", "step_us", "step_us_regions",
+    "bound_eager_step_us", "graph_step_us", "per_rank_api_step_us", "per_rank_api_calls_per_step", "dispatch_us",
+    "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac", "graph_replay_1000x_us",
+    "graph_replay_1000x_note",
 )  # fmt: skip
+
+
+def compact(res):
+    return {k: res[k] for k in COMPACT_FIELDS if k in res}
 
 
 def main() -> None:
@@ -384,24 +444,29 @@ def main() -> None:
     del steps
     torch.cuda.empty_cache()
 
-    workloads = {args.workload: {k: main_res[k] for k in COMPACT_FIELDS}}
+    workloads = {args.workload: compact(main_res)}
+    if not args.no_cpu:
+        workloads[args.workload]["cpu_baseline"] = cpu_baseline(spec, groups)
+    del groups
     if not args.only:
         # the 8192-token prefill (the >= 60 % target) first, then the rest
         for name in ("C5", "C4", "C3", "C1"):
             if name == args.workload:
                 continue
-            res, _, st = measure_workload(name, specs[name], steps_for(name, args.steps), min(args.warmup, 5))
+            res, grp, st = measure_workload(name, specs[name], steps_for(name, args.steps), min(args.warmup, 5))
             del st
             torch.cuda.empty_cache()
-            workloads[name] = {k: res[k] for k in COMPACT_FIELDS}
-            if name == "C1" and not args.no_cpu:
-                workloads[name]["cpu_literal_loops"] = cpu_literal_loops(specs[name])
+            workloads[name] = compact(res)
+            if not args.no_cpu:
+                workloads[name]["cpu_baseline"] = cpu_baseline(specs[name], grp)
+                if name == "C1":
+                    workloads[name]["cpu_literal_loops"] = cpu_literal_loops(specs[name])
+            del grp
 
-    form = {
-        "bound_eager": "eager launches of a bound step (LoopbackWorld.bind: pplx_a2a_world_dispatch + _combine on "
-        "arguments packed once)",
-        "graph_replay": f"one captured hipGraph replayed {GRAPH_REPLAYS_C3} times",
-    }[main_res["launch_form"]]
+    form = (
+        "eager launches of a bound step (LoopbackWorld.bind: pplx_a2a_world_dispatch + _combine on arguments "
+        "packed once)"
+    )
     result = {
         "metric": "dispatch+combine latency (us) and achieved HBM GB/s, DSv3 shape 128 tok/rank, 1 GPU",
         "value": main_res["step_us"],
@@ -425,14 +490,16 @@ def main() -> None:
             "in_dtype": str(spec.in_dtype).replace("torch.", ""),
             "out_dtype": str(spec.out_dtype).replace("torch.", ""),
             "timed": f"{form}, rotating buffer sets; the same step as a hipGraph replay takes "
-            f"{main_res['graph_step_us']:.1f} us, as bound eager launches {main_res['bound_eager_step_us']:.1f} us",
+            f"{main_res['graph_step_us']:.1f} us, through the reference's per-rank API "
+            f"(AllToAll.dispatch / .combine, {main_res['per_rank_api_calls_per_step']} calls) "
+            f"{main_res['per_rank_api_step_us']:.1f} us",
         },
         "roofline": roofline,
         "workloads": workloads,
         "detail": main_res,
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(spec, groups)
+        result["cpu_baseline"] = workloads[args.workload]["cpu_baseline"]
     print(json.dumps(result))
 
 
