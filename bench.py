@@ -387,6 +387,52 @@ def counter_probe(spec, launches=3):
     world.destroy()
 
 
+TIMELINE_PHASES = (
+    "workgroup entered", "rank table in LDS", "earlier picks counted", "own picks marked, row loads issued",
+    "barrier passed", "slots and destinations resolved", "row arrived", "stores issued", "stores complete",
+)  # fmt: skip
+
+
+def fused_dispatch_timeline(spec, launches=6):
+    """Per-workgroup phase times of the one-launch dispatch, from a library built with
+    `make -C pplx-kernels_amd/csrc -B TIMELINE=1`: thread 0 of every workgroup stamps the GPU's
+    100 MHz clock at its phase boundaries.  Each launch is made cold (a 768 MB fill in front evicts
+    the caches); the last three are summarised as ns after the first workgroup's entry."""
+    import ctypes
+
+    import numpy as np
+
+    from pplx_kernels import ops
+    from pplx_kernels.workloads import DeviceStep, generate, make_world
+
+    lib = ops.load_library()
+    if not hasattr(lib, "pplx_a2a_debug_timeline"):
+        sys.exit("bench.py --timeline needs a library built with `make -C pplx-kernels_amd/csrc -B TIMELINE=1`")
+    lib.pplx_a2a_debug_timeline.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    step = DeviceStep(spec, generate(spec))
+    world = make_world(spec, group_name="timeline")
+    evict = torch.empty(768 << 20, dtype=torch.uint8, device="cuda")
+    print(f"dispatch_fused phase times, workload {spec.name}, library build {lib.pplx_a2a_build_id().decode()} + TIMELINE")
+    for it in range(launches):
+        evict.fill_(it)
+        torch.cuda.synchronize()
+        step.dispatch_world(world)
+        torch.cuda.synchronize()
+        buf = (ctypes.c_ulonglong * 16384)()
+        assert lib.pplx_a2a_debug_timeline(buf, 16384) == 0
+        a = np.frombuffer(buf, dtype=np.uint64).reshape(1024, 16).astype(np.int64)
+        a = a[: int((a[:, 0] > 0).sum())]
+        rel = (a[:, :9] - a[:, 0].min()) * 10
+        if it < launches - 3:
+            continue
+        print(f"launch {it}: {len(a)} workgroups, last store complete {rel[:, 8].max()} ns after the first entry")
+        print(f"  {'phase':<38s} {'min':>7s} {'median':>7s} {'p90':>7s} {'max':>7s}  ns")
+        for i, label in enumerate(TIMELINE_PHASES):
+            col = rel[:, i]
+            print(f"  {label:<38s} {col.min():7d} {int(np.median(col)):7d} {int(np.percentile(col, 90)):7d} {col.max():7d}")
+    world.destroy()
+
+
 def steps_for(name, steps_k):
     """Timed steps per workload: the large prefills take milliseconds per step."""
     if name == "C5":
@@ -418,6 +464,7 @@ def main() -> None:
     ap.add_argument("--all", action="store_true", help="accepted for compatibility: every workload is measured by default")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-probe", action="store_true", help="few eager launches + a calibration copy, for rocprofv3 --pmc")
+    ap.add_argument("--timeline", action="store_true", help="phase times of the one-launch dispatch (needs a TIMELINE=1 build)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(
@@ -438,6 +485,9 @@ def main() -> None:
     spec = specs[args.workload]
     if args.counter_probe:
         counter_probe(spec)
+        return
+    if args.timeline:
+        fused_dispatch_timeline(spec)
         return
     main_res, groups, steps = measure_workload(args.workload, spec, steps_for(args.workload, args.steps), args.warmup)
     roofline = combine_kernel_roofline(args.workload, spec, steps, main_res["combine_bytes"], args.steps)

@@ -30,8 +30,36 @@
 #include "a2a_route.h"
 #include "a2a_rows.h"
 
+// Built with -DPPLX_A2A_TIMELINE (make TIMELINE=1), dispatch_fused records when thread 0 of every
+// workgroup passes its phase boundaries (the GPU's 100 MHz wall clock) into a table that
+// pplx_a2a_debug_timeline copies out; `bench.py --timeline` prints the summary.  The waits that
+// the stamps need (for the row, for the stores) are not in the regular build.
+#ifdef PPLX_A2A_TIMELINE
+__device__ unsigned long long g_timeline[1024 * 16];
+extern "C" int pplx_a2a_debug_timeline(unsigned long long *host, int words) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_timeline), sizeof(unsigned long long) * (size_t)words);
+}
+#endif
+
 namespace pplx_amd {
 namespace {
+
+struct Timeline {
+#ifdef PPLX_A2A_TIMELINE
+  unsigned long long at[9];
+  __device__ __forceinline__ void mark(int i) { at[i] = wall_clock64(); }
+  __device__ __forceinline__ void wait_for_memory() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+  __device__ __forceinline__ void flush() {
+    if (threadIdx.x != 0 || blockIdx.x >= 1024) return;
+    for (int i = 0; i < 9; ++i) g_timeline[blockIdx.x * 16 + i] = at[i];
+    g_timeline[blockIdx.x * 16 + 9] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11)) & 0xf;  // XCC id
+  }
+#else
+  __device__ __forceinline__ void mark(int) {}
+  __device__ __forceinline__ void wait_for_memory() {}
+  __device__ __forceinline__ void flush() {}
+#endif
+};
 
 // ---------------------------------------------------------------------------
 // Table binding: rows arrive as kernel arguments and are stored with vector
@@ -216,6 +244,8 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
                                                                   uint8_t *stage) {
   constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
+  Timeline timeline;
+  timeline.mark(0);
   constexpr bool kStaged = DT::kInline;
   constexpr uint32_t kRowWords = sizeof(DispatchRank) / 8;
   const uint32_t table_words = kStaged ? w.R * kRowWords : 0;
@@ -228,6 +258,7 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   for (uint32_t e = threadIdx.x; e < 2 * w.E; e += kFusedThreads) hist[e] = 0;
   // Orders the zeroing (and the staged table) before the first counter update of any wave.
   __syncthreads();
+  timeline.mark(1);
   const LdsDispatch staged{reinterpret_cast<const DispatchRank *>(lds_u64)};
   auto rows = [&]() -> decltype(auto) {
     if constexpr (kStaged) return (staged); else return (tab);
@@ -261,6 +292,7 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   } else {
     count_earlier_picks<1, kFusedThreads>(w, rows(), v0, hist);
   }
+  timeline.mark(2);
   // ... and the workgroup's own: a pick that names no expert, or repeats an earlier pick of its
   // token, has no row.
   uint32_t my_n = my_bounded ? my_loaded_n : my_head.m;
@@ -274,9 +306,11 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   }
   const bool my_pick_has_row = my_live && my_e < w.E && !my_repeats;
   if (my_pick_has_row && my_part == 0) atomicOr(&own_mask[my_e], 1u << my_j);
+  timeline.mark(3);
   RowRegs<NV> regs;
   if (my_live) load_row<NV, EXACT>(w, my_src, my_t, lane, regs);
   __syncthreads();
+  timeline.mark(4);
 
   // 3. own slots and destinations
   uint32_t my_slot = kInvalidSlot;
@@ -321,8 +355,11 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
     }
   }
 
+  timeline.mark(5);
   // 4. fan out
   if (my_live) {
+    timeline.wait_for_memory();
+    timeline.mark(6);
     const uint32_t k0 = my_part * kper;
     const uint32_t k1 = (k0 + kper < w.K) ? k0 + kper : w.K;
     if (write_through) {
@@ -331,6 +368,10 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
       store_row<NV, EXACT, RowStore::kStream>(w, my_src, my_t, lane, dst, k0, k1, regs);
     }
   }
+  timeline.mark(7);
+  timeline.wait_for_memory();
+  timeline.mark(8);
+  timeline.flush();
   // A bound_m beyond the limit is reported once, behind the stores (it costs a trip to memory).
   if (blockIdx.x == 0) {
     for (uint32_t g = threadIdx.x; g < w.G; g += kFusedThreads) {

@@ -5,7 +5,8 @@ shapes, :252-268; same event-timed loop: 10 samples per run, 10 warm-up runs, 20
 mean and standard deviation; same one-way payload formulas, :131-139).  All simulated ranks live
 in this process, so one "dispatch" below is the sum of every rank's call, launched from the
 host without a graph: it measures what a caller of the reference API sees, Python included.
-``bench.py`` at the repository root measures the kernels themselves (hipGraph replay).
+``bench.py`` at the repository root measures the workloads of the benchmark plan in every
+launch form (its ``per_rank_api_step_us`` is this path on those workloads).
 
     python -m tests.bench_all_to_all [--ranks 8] [--dp-size 1] [--in-dtype float8_e4m3fn]
 """
@@ -84,7 +85,11 @@ def main() -> None:
     ap.add_argument("--dp-size", type=int, default=1)
     ap.add_argument("--in-dtype", default="float8_e4m3fn", choices=["bfloat16", "float16", "float8_e4m3fn"])
     ap.add_argument("--out-dtype", default="bfloat16", choices=["bfloat16", "float16"])
+    ap.add_argument("--quick", action="store_true", help="two token counts per model, fewer runs")
     args = ap.parse_args()
+    global TOKENS, WARMUP_RUNS, MEASURED_RUNS
+    if args.quick:
+        TOKENS, WARMUP_RUNS, MEASURED_RUNS = [1, 128], 2, 4
     if not torch.cuda.is_available():
         sys.exit("bench_all_to_all: no GPU visible")
     in_dtype, out_dtype = getattr(torch, args.in_dtype), getattr(torch, args.out_dtype)

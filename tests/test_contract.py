@@ -490,3 +490,30 @@ def test_cpp_memory_yardstick_runs():
     rates = [float(line.split("TB/s")[0].split()[-1]) for line in proc.stdout.splitlines() if "TB/s " in line]
     assert len(rates) == 15
     assert all(0.8 < r < 8.0 for r in rates), rates
+
+
+def test_cpp_launch_floor_runs():
+    """The launch-cost yardstick (empty kernels, eager and as graph replays) that the latency of
+    the decode-sized steps is read against: four lines of eight finite figures."""
+    exe = os.path.join(ROOT, "pplx-kernels_amd", "bin", "bench_launch")
+    assert os.path.exists(exe), "build it with `make -C pplx-kernels_amd/csrc`"
+    proc = subprocess.run([exe, "300"], capture_output=True, text=True, timeout=300)
+    print(proc.stdout[-3000:], proc.stderr[-2000:])
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    rows = [line.split()[-8:] for line in proc.stdout.splitlines() if "of arguments" in line]
+    assert len(rows) == 4
+    assert all(0.05 < float(x) < 1000.0 for row in rows for x in row), rows
+
+
+def test_per_rank_api_benchmark_prints_its_table():
+    """tests/bench_all_to_all.py (the eager per-rank latency table, counterpart of the reference's
+    tests/bench_all_to_all.py) runs to the end for a small rank count."""
+    import sys
+
+    proc = subprocess.run(
+        [sys.executable, "-m", "tests.bench_all_to_all", "--ranks", "4", "--quick"],
+        capture_output=True, text=True, timeout=300, cwd=ROOT,
+    )  # fmt: skip
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    lines = [line for line in proc.stdout.splitlines() if line[:1].isdigit()]
+    assert len(lines) >= 4 and all("GB/s" in line for line in lines), proc.stdout[-2000:]
