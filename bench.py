@@ -19,6 +19,12 @@ launch forms under fixed keys, on the same rotating buffer sets:
   simulated rank and then ``AllToAll.combine`` once per rank, eagerly, arguments checked on
   every call (what ``tests/bench_all_to_all.py`` of the reference times per rank).
 
+``bound_eager_host_us_per_call`` is what the launching thread spends on one of those library
+calls (issued into an empty queue).  Every timed region is exactly ``--steps`` steps between two
+synchronisations; in front of it come at least 64 untimed calls (more if ``--warmup`` says so)
+and, behind the synchronisation, 200 us of busy host, so that a region of 20 decode steps is not
+dominated by a thread that has just woken up (see ``wake_host``).
+
 The decode shape C3 additionally carries ``graph_replay_1000x_us``: ONE captured graph over ONE
 buffer set replayed 1000 times, the form its specification names; 12.5 MB replayed back to back
 stay in the last-level cache, so that figure is cache-resident and carries no HBM fraction.
@@ -95,15 +101,35 @@ def build_steps(spec, groups, cap, n_sets):
     return steps
 
 
+HOST_WAKE_US = 200.0
+# Untimed calls in front of every timed region, whatever --warmup says: every buffer set (up to
+# eight) is touched several times and the launch path of the host is warm before 20 steps of
+# 10 us each are timed.
+MIN_WARMUP_CALLS = 64
+
+
+def wake_host():
+    """Keeps the launching thread busy for a moment between the synchronisation in front of a
+    timed region and its first launch.  A blocking wait parks the thread, and the launches it
+    issues right after waking are two to three times slower than in a running loop; a region of
+    20 decode steps (0.2 ms, two launches of host-bound size each) cannot amortise that: without
+    this, 20-step regions of C3 read 11.2-18.5 us per step, with it 10.5-10.9, as 200-step
+    regions do.  Steps whose kernels outlast the host's part of a launch do not notice."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e6 < HOST_WAKE_US:
+        pass
+
+
 def time_graphs(graphs, order, stream, warmup, repeats=1):
     """Mean microseconds per graph launch over `order` (a list of graph indices), HIP events
     on the launch stream."""
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
-        for i in range(warmup):
+        for i in range(max(warmup, MIN_WARMUP_CALLS)):
             graphs[order[i % len(order)]].replay(stream)
         stream.synchronize()
         torch.cuda.synchronize()
+        wake_host()
         start.record(stream)
         for _ in range(repeats):
             for i in order:
@@ -119,15 +145,33 @@ def time_steps(run, order, stream, warmup):
     HIP events on the launch stream, which is also the current stream inside run."""
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
-        for i in range(warmup):
+        for i in range(max(warmup, MIN_WARMUP_CALLS)):
             run(order[i % len(order)])
         stream.synchronize()
+        wake_host()
         start.record(stream)
         for i in order:
             run(i)
         end.record(stream)
         stream.synchronize()
     return start.elapsed_time(end) * 1e3 / len(order)
+
+
+def host_cost(run, n_sets, stream, calls=16):
+    """Host microseconds per call of run(i), issued into an empty queue (the launches are
+    asynchronous: this is what the launching thread spends, whatever the kernels take)."""
+    best = None
+    with torch.cuda.stream(stream):
+        for _ in range(5):
+            stream.synchronize()
+            wake_host()
+            t0 = time.perf_counter()
+            for i in range(calls):
+                run(i % n_sets)
+            t = (time.perf_counter() - t0) * 1e6 / calls
+            best = t if best is None else min(best, t)
+        stream.synchronize()
+    return best
 
 
 def capture(world, stream, body):
@@ -170,6 +214,7 @@ def measure_workload(name, spec, steps_k, warmup):
         time_steps(lambda i: (bound[i].dispatch(stream), bound[i].combine(stream)), order, stream, 0)
         for _ in range(EXTRA_REGIONS)
     ]
+    host_us = host_cost(lambda i: (bound[i].dispatch(stream), bound[i].combine(stream)), n_sets, stream) / 2
     d_us = time_steps(lambda i: bound[i].dispatch(stream), order, stream, warmup)
     c_us = time_steps(lambda i: bound[i].combine(stream), order, stream, warmup)
 
@@ -213,6 +258,7 @@ def measure_workload(name, spec, steps_k, warmup):
             "note": f"{len(spread)} timed regions of {len(order)} steps each; step_us is the first",
         },
         "bound_eager_step_us": bound_us,
+        "bound_eager_host_us_per_call": host_us,
         "graph_step_us": graph_us,
         "per_rank_api_step_us": per_rank_us,
         "per_rank_api_calls_per_step": 2 * spec.world_size,
@@ -444,7 +490,7 @@ def steps_for(name, steps_k):
 
 COMPACT_FIELDS = (
     "workload", "tokens", "pairs", "buffer_sets", "steps_timed", "launch_form", "step_us", "step_us_regions",
-    "bound_eager_step_us", "graph_step_us", "per_rank_api_step_us", "per_rank_api_calls_per_step", "dispatch_us",
+    "bound_eager_step_us", "bound_eager_host_us_per_call", "graph_step_us", "per_rank_api_step_us", "per_rank_api_calls_per_step", "dispatch_us",
     "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac", "graph_replay_1000x_us",
     "graph_replay_1000x_note",
 )  # fmt: skip
