@@ -263,3 +263,22 @@ def test_no_kernel_spills_or_uses_scratch():
         if k[".private_segment_fixed_size"] or k.get(".vgpr_spill_count", 0) or k.get(".sgpr_spill_count", 0)
     ]
     assert not offenders, offenders
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every simulated rank shares one GPU's HBM: `bench.py --gpus N` with N above 1 (or under a
+    launcher that sets WORLD_SIZE) exits with a message that says so, before it touches a GPU."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ)
+    env.pop("WORLD_SIZE", None)
+    for argv, extra in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "8"})):
+        done = subprocess.run(
+            [sys.executable, os.path.join(root, "bench.py"), *argv],
+            env={**env, **extra}, capture_output=True, text=True, timeout=120,
+        )  # fmt: skip
+        assert done.returncode == 2, done
+        assert "single-GPU loopback" in done.stderr and "--gpus 1" in done.stderr
+        assert done.stdout == ""
