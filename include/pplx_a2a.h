@@ -165,7 +165,14 @@ uint32_t pplx_a2a_rank(const pplx_a2a_t *handle);
  * SEND and RECV are collective in the same way, phase by phase: the last
  * rank's SEND enqueues the sends of all ranks (inputs may be reused once it has
  * returned, in stream order; no output is touched), the last rank's RECV the
- * receives (outputs are those named by the RECV calls).  Every rank's SEND must
+ * receives (outputs are those named by the RECV calls).  A SEND takes over
+ * everything its call's inputs hold: dispatch SEND copies every present token
+ * (row, scales, picks) and the groups' token counts into the staging area and
+ * RECV routes and places them; combine SEND reads expert_y, indices, weights
+ * and bound_m and leaves the combined rows in the staging area, and RECV copies
+ * them to out_tokens (the reference reads indices and weights in its RECV,
+ * csrc/all_to_all/intranode_combine.cu:127-169: pass the same ones to both
+ * calls, as its callers do).  Every rank's SEND must
  * come before the first RECV, and staging must have been reserved with
  * pplx_a2a_world_reserve_split (PPLX_A2A_INVALID_STATE otherwise).
  * Without bound_m, m may not exceed max_num_tokens
@@ -238,14 +245,16 @@ pplx_a2a_world_t *pplx_a2a_world_of(const pplx_a2a_t *handle);
 
 /* Allocates the staging that split send / recv calls go through (the reference
  * allocates its inboxes in the constructor, csrc/all_to_all/intranode.cpp:37-136;
- * here a world that never splits does not pay for them): about
- * G*M*K * (hidden_dim_bytes + hidden_dim_scale_bytes + 16) bytes for dispatch plus
- * G*M*K * hidden_dim * expert_y_elem_bytes for combine (0 = dispatch only, 2 =
- * bf16 / f16 expert_y, 4 = also f32).  May be called again with a wider element
- * while no split combine step is in flight, which frees the narrower combine staging: once a
- * stream capture has recorded split calls of the world the graph holds that address, and a
- * widening call returns PPLX_A2A_INVALID_STATE (reserve the widest element before capturing).
- * Synchronises the device. */
+ * here a world that never splits does not pay for them).  With G = world_size /
+ * dp_size DP groups and M = max_num_tokens: G*M * (hidden_dim_bytes +
+ * hidden_dim_scale_bytes + 4 * experts_per_token) bytes for dispatch (one copy
+ * of every token, its scales and its picks) and, when expert_y_elem_bytes is not
+ * 0, world_size*M * hidden_dim * 2 bytes for combine (one combined row per rank
+ * and token, in the 2-byte dtype of out_tokens whatever expert_y holds; 2 and 4
+ * ask for the same).  May be called again: what has been allocated stays where
+ * it is until the world is destroyed, so graphs that recorded split calls remain
+ * valid.  The first call (and the first that asks for combine staging)
+ * allocates and clears memory, which synchronises the device. */
 int pplx_a2a_world_reserve_split(pplx_a2a_world_t *world, uint32_t expert_y_elem_bytes);
 
 /* Reads and clears the world's device-side fault word (synchronises `stream`):

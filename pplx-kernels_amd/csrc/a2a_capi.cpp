@@ -131,13 +131,9 @@ struct pplx_a2a_world {
   // record which ranks have made which call of the step in flight.
   SplitDev split{};
   bool split_ready = false;
-  uint32_t split_y_elem_bytes = 0;  // widest expert_y element the combine staging holds
   std::vector<uint8_t> dsend, drecv, csend, crecv;
   uint32_t n_dsend = 0, n_drecv = 0, n_csend = 0, n_crecv = 0;
-  int split_in_dtype = -1;
-  // A stream capture has recorded split-mode kernels: the graph holds the staging addresses as
-  // kernel arguments, so the staging may no longer move.
-  bool split_captured = false;
+  int split_in_dtype = -1, split_out_dtype = -1;  // dtypes of the combine SEND phase in flight
 };
 
 struct pplx_a2a {
@@ -486,14 +482,15 @@ int run_combine(pplx_a2a_world &w, void *stream) {
 
 void free_split(pplx_a2a_world &w) {
   SplitDev &sp = w.split;
-  (void)hipFree(sp.stage_x);  // gexp and gcnt live behind the rows
+  (void)hipFree(sp.stage_x);  // the picks and the groups' counts live behind the rows
   (void)hipFree(sp.stage_y);
   sp = SplitDev{};
   w.split_ready = false;
-  w.split_y_elem_bytes = 0;
 }
 
-// Allocates (or widens) the staging of split mode.  Never part of a dispatch / combine call.
+// Allocates the staging of split mode: the tokens' area on the first call, the combined rows'
+// area on the first call that asks for it.  Never part of a dispatch / combine call; nothing
+// that has been allocated moves or is freed before the world goes.
 int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
   if (y_elem_bytes != 0 && y_elem_bytes != 2 && y_elem_bytes != 4)
     return fail(PPLX_A2A_INVALID_ARGUMENT, "expert_y_elem_bytes must be 0, 2 or 4");
@@ -501,11 +498,10 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
   if (!scope.ok()) return fail(PPLX_A2A_HIP_ERROR, "cannot select device %d", w.device);
   const WorldDev &d = w.dev;
   SplitDev &sp = w.split;
-  const size_t pairs = (size_t)d.G * d.M * d.K;
   if (!w.split_ready) {
     if (w.n_arrived_dispatch != 0 || w.n_arrived_combine != 0)
       return fail(PPLX_A2A_INVALID_STATE, "a step is being assembled");
-    const StageLayout lay = stage_layout(d.Hb, d.S, pairs, d.E);
+    const StageLayout lay = stage_layout(d.Hb, d.S, (uint64_t)d.G * d.M, d.K, d.G);
     hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_x), lay.bytes);
     if (err == hipSuccess) err = hipMemset(sp.stage_x, 0, lay.bytes);
     if (err != hipSuccess) {
@@ -514,44 +510,32 @@ int reserve_split(pplx_a2a_world &w, uint32_t y_elem_bytes) {
                   hipGetErrorString(err));
     }
     sp.token_stride = lay.token_stride;
-    sp.gexp = reinterpret_cast<uint32_t *>(sp.stage_x + lay.gexp_offset);
-    sp.gcnt = reinterpret_cast<uint32_t *>(sp.stage_x + lay.gcnt_offset);
+    sp.stage_idx = reinterpret_cast<uint32_t *>(sp.stage_x + lay.idx_offset);
+    sp.stage_n = reinterpret_cast<uint32_t *>(sp.stage_x + lay.n_offset);
     w.dsend.assign(d.R, 0);
     w.drecv.assign(d.R, 0);
     w.csend.assign(d.R, 0);
     w.crecv.assign(d.R, 0);
     w.split_ready = true;
   }
-  if (y_elem_bytes > w.split_y_elem_bytes) {
-    if (w.n_csend != 0 || w.n_crecv != 0)
-      return fail(PPLX_A2A_INVALID_STATE, "a split combine step is in flight");
-    // Widening frees the old combine staging.  A graph that recorded split calls carries its
-    // address and would write through it on the next replay.
-    if (w.split_captured && w.split.stage_y != nullptr)
-      return fail(PPLX_A2A_INVALID_STATE,
-                  "split calls of this world have been captured into a graph, which holds the address of the "
-                  "combine staging: it cannot be widened to %u-byte elements any more (reserve the widest "
-                  "expert_y element before capturing)", y_elem_bytes);
-    // stage_y holds one expert_y row per (token, pick)
-    HIP_TRY(hipDeviceSynchronize());
-    (void)hipFree(sp.stage_y);
-    sp.stage_y = nullptr;
-    w.split_y_elem_bytes = 0;
-    const size_t bytes = pairs * (size_t)d.H * y_elem_bytes;
+  if (y_elem_bytes != 0 && sp.stage_y == nullptr) {
+    // one combined row per (rank, token); out_tokens has 2-byte elements whatever expert_y has
+    const size_t bytes = (size_t)d.R * d.M * d.H * 2u;
     hipError_t err = hipMalloc(reinterpret_cast<void **>(&sp.stage_y), bytes);
-    if (err != hipSuccess)
+    if (err != hipSuccess) {
+      sp.stage_y = nullptr;
       return fail(PPLX_A2A_HIP_ERROR, "allocating %zu bytes of combine staging failed: %s", bytes,
                   hipGetErrorString(err));
-    w.split_y_elem_bytes = y_elem_bytes;
+    }
   }
   return PPLX_A2A_OK;
 }
 
-int need_split(const pplx_a2a_world &w, uint32_t y_elem_bytes) {
-  if (!w.split_ready || w.split_y_elem_bytes < y_elem_bytes)
+int need_split(const pplx_a2a_world &w, bool combine) {
+  if (!w.split_ready || (combine && w.split.stage_y == nullptr))
     return fail(PPLX_A2A_INVALID_STATE,
-                "send / recv calls need staging for %u-byte expert_y elements: call "
-                "pplx_a2a_world_reserve_split first (dispatch and combine never allocate)", y_elem_bytes);
+                "send / recv calls need staging%s: call pplx_a2a_world_reserve_split first (dispatch and "
+                "combine never allocate)", combine ? " for combine (a non-zero expert_y_elem_bytes)" : "");
   return PPLX_A2A_OK;
 }
 
@@ -566,21 +550,40 @@ int run_split_dispatch(pplx_a2a_world &w, int mode, void *stream) {
   int st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_dispatch, w.bound_dispatch_valid);
-  if (session != 0) w.split_captured = true;
-  const DispatchRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_dispatch.data() : nullptr;
+  const WorldDev &d = w.dev;
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    st = check_groups(d, w.pend_dispatch.data());
+    if (st) return st;
+  } else {
+    // RECV is the one-call dispatch on what SEND staged: every rank's inputs are its DP
+    // group's part of the staging area, its outputs those of its RECV call.
+    const SplitDev &sp = w.split;
+    for (uint32_t r = 0; r < d.R; ++r) {
+      const uint32_t g = r / d.dp;
+      DispatchRank &row = w.pend_dispatch[r];
+      const uint8_t *rows = sp.stage_x + (uint64_t)g * d.M * sp.token_stride;
+      row.dp_x = rows;
+      row.dp_x_stride_row = sp.token_stride;
+      row.dp_xs = d.S ? reinterpret_cast<const float *>(rows + d.Hb) : nullptr;
+      row.dp_xs_stride_elem = 1;
+      row.dp_xs_stride_row = sp.token_stride / 4;
+      row.indices = sp.stage_idx + (uint64_t)g * d.M * d.K;
+      row.bound_m = sp.stage_n + g;
+      row.m = d.M;
+    }
+  }
+  const DispatchRank *inline_rows = d.R <= kInlineRanks ? w.pend_dispatch.data() : nullptr;
   if (!inline_rows) {
     st = flush_table<DispatchRank, BindDispatchBatch>(w, w.pend_dispatch, w.bound_dispatch,
                                                       w.bound_dispatch_valid, false, launch_bind_dispatch, stream);
     if (st) return st;
   }
   if (mode == PPLX_A2A_SPLIT_SEND) {
-    st = check_groups(w.dev, w.pend_dispatch.data());
-    if (st) return st;
     ProfilerRange range("dispatch send");
-    LAUNCH_TRY(launch_split_dispatch_send(w.dev, w.split, inline_rows, pick_vector_of(w), stream));
+    LAUNCH_TRY(launch_split_stage_tokens(d, w.split, inline_rows, stream));
   } else {
     ProfilerRange range("dispatch recv");
-    LAUNCH_TRY(launch_split_dispatch_recv(w.dev, w.split, inline_rows, stream));
+    LAUNCH_TRY(launch_dispatch(d, inline_rows, pick_vector_of(w), stream));
   }
   return PPLX_A2A_OK;
 }
@@ -588,7 +591,7 @@ int run_split_dispatch(pplx_a2a_world &w, int mode, void *stream) {
 int split_dispatch(pplx_a2a_world &w, uint32_t rank, const DispatchRank &row, int mode, void *stream) {
   if (w.n_arrived_dispatch != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv dispatch step is still being assembled");
-  int st = need_split(w, 0);
+  int st = need_split(w, false);
   if (st) return st;
   const uint32_t R = w.dev.R;
   if (mode == PPLX_A2A_SPLIT_SEND) {
@@ -629,8 +632,16 @@ int run_split_combine(pplx_a2a_world &w, int mode, int in_dtype, int out_dtype, 
   int st = capture_session(stream, &session);
   if (st) return st;
   settle_mirror(w, session, w.bind_capture_combine, w.bound_combine_valid);
-  if (session != 0) w.split_captured = true;
-  const CombineRank *inline_rows = w.dev.R <= kInlineRanks ? w.pend_combine.data() : nullptr;
+  const WorldDev &d = w.dev;
+  if (mode == PPLX_A2A_SPLIT_SEND) {
+    // SEND is the one-call combine with every rank's output rows in the staging area.
+    for (uint32_t r = 0; r < d.R; ++r) {
+      CombineRank &row = w.pend_combine[r];
+      row.out_tokens = w.split.stage_y + (uint64_t)r * d.M * d.H * 2u;
+      row.out_stride_row = d.H;
+    }
+  }
+  const CombineRank *inline_rows = d.R <= kInlineRanks ? w.pend_combine.data() : nullptr;
   if (!inline_rows) {
     st = flush_table<CombineRank, BindCombineBatch>(w, w.pend_combine, w.bound_combine, w.bound_combine_valid,
                                                     false, launch_bind_combine, stream);
@@ -638,10 +649,10 @@ int run_split_combine(pplx_a2a_world &w, int mode, int in_dtype, int out_dtype, 
   }
   if (mode == PPLX_A2A_SPLIT_SEND) {
     ProfilerRange range("combine send");
-    LAUNCH_TRY(launch_split_combine_send(w.dev, w.split, inline_rows, in_dtype, stream));
+    LAUNCH_TRY(launch_combine(d, inline_rows, in_dtype, out_dtype, stream));
   } else {
     ProfilerRange range("combine recv");
-    LAUNCH_TRY(launch_split_combine_recv(w.dev, w.split, inline_rows, in_dtype, out_dtype, stream));
+    LAUNCH_TRY(launch_split_deliver(d, w.split, inline_rows, stream));
   }
   return PPLX_A2A_OK;
 }
@@ -650,7 +661,7 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
                   int mode, void *stream) {
   if (w.n_arrived_combine != 0)
     return fail(PPLX_A2A_INVALID_STATE, "a send+recv combine step is still being assembled");
-  int st = need_split(w, (uint32_t)dtype_size(in_dtype));
+  int st = need_split(w, true);
   if (st) return st;
   const uint32_t R = w.dev.R;
   if (mode == PPLX_A2A_SPLIT_SEND) {
@@ -658,10 +669,10 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
       return fail(PPLX_A2A_INVALID_STATE,
                   "rank %u: combine SEND of the next step before every rank's RECV of this one", rank);
     if (w.csend[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine SEND twice", rank);
-    if (w.n_csend != 0 && w.split_in_dtype != in_dtype)
+    if (w.n_csend != 0 && (w.split_in_dtype != in_dtype || w.split_out_dtype != out_dtype))
       return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
     w.split_in_dtype = in_dtype;
-    w.split.y_row_bytes = (uint64_t)w.dev.H * dtype_size(in_dtype);
+    w.split_out_dtype = out_dtype;
     w.pend_combine[rank] = row;
     w.stream_combine[rank] = stream;
     w.csend[rank] = 1;
@@ -679,11 +690,9 @@ int split_combine(pplx_a2a_world &w, uint32_t rank, const CombineRank &row, int 
                 "rank %u: combine RECV before every rank's SEND (%u of %u sent); in a loopback "
                 "world all SENDs must be enqueued first", rank, w.n_csend, R);
   if (w.crecv[rank]) return fail(PPLX_A2A_INVALID_STATE, "rank %u called combine RECV twice", rank);
-  if (w.split_in_dtype != in_dtype)
-    return fail(PPLX_A2A_UNSUPPORTED, "combine RECV must use the expert_y dtype of the SEND phase");
-  if (w.n_crecv != 0 && w.combine_out_dtype != out_dtype)
-    return fail(PPLX_A2A_UNSUPPORTED, "all ranks of a step must combine with the same dtypes");
-  w.combine_out_dtype = out_dtype;
+  // (the rows were combined, and converted to the out_tokens dtype, by the SEND phase)
+  if (w.split_in_dtype != in_dtype || w.split_out_dtype != out_dtype)
+    return fail(PPLX_A2A_UNSUPPORTED, "combine RECV must use the dtypes of the SEND phase");
   w.pend_combine[rank] = row;
   w.stream_combine[rank] = stream;
   w.crecv[rank] = 1;

@@ -1,5 +1,5 @@
 // gfx950 combine kernel of the MoE dispatch / combine path: the top-k weighted
-// gather-reduce, for expert_y in place (one-call mode) or for the staged rows of split mode.
+// gather-reduce (also the SEND phase of a split combine, with its output rows in the staging area).
 #include "a2a_common.h"
 
 namespace pplx_amd {
@@ -93,8 +93,7 @@ __device__ __forceinline__ void gather_group(f32x8 (&acc)[VPL], uint64_t row_of_
 // picks read long pieces of their rows, many picks shorter ones.
 template <typename T, typename U, class CT, int KB, int VPL>
 __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32_t segments, FastDiv by_segments,
-                                                      uint32_t first_rank, uint32_t rank_count,
-                                                      const uint8_t *stage_y, uint64_t stage_row_bytes) {
+                                                      uint32_t first_rank, uint32_t rank_count) {
   const uint32_t lane = lane_id();
   const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) +
                                                        threadIdx.x / kWave);
@@ -114,13 +113,7 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
     const uint32_t e = as_global(c.indices)[(size_t)t * w.K + lane];
     const uint32_t slot = as_global(w.slot_map)[((size_t)fast_div(r, w.by_dp) * w.M + t) * w.K + lane];
     weight = as_global(c.weights)[(int64_t)t * c.w_stride_row + lane];
-    if (CT::kStaged) {
-      // combine SEND left the row of (token, pick) in the staging area.
-      if (e < w.E && slot != kInvalidSlot) {
-        row = reinterpret_cast<uint64_t>(stage_y) +
-              (((uint64_t)fast_div(r, w.by_dp) * w.M + t) * w.K + lane) * stage_row_bytes;
-      }
-    } else if (e < w.E && slot != kInvalidSlot) {
+    if (e < w.E && slot != kInvalidSlot) {
       const CombineRank &owner = tab.at(owner_of(w, e));
       if (slot < owner.y_rows) {
         row = reinterpret_cast<uint64_t>(reinterpret_cast<const T *>(owner.expert_y) +
@@ -176,33 +169,29 @@ __global__ __launch_bounds__(256) void combine_gather(WorldDev w, CT tab, uint32
 }
 
 template <typename T, typename U, class CT, int KB, int VPL>
-int launch_combine_v(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
-                     const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
+int launch_combine_v(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count, hipStream_t s) {
   const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
   const uint32_t segments = (nvec_segments + VPL - 1) / VPL;
   const uint64_t waves = (uint64_t)rank_count * w.M * segments;
   const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
   hipLaunchKernelGGL((combine_gather<T, U, CT, KB, VPL>), grid, block, 0, s, w, tab, segments,
-                     make_fast_div(segments), first_rank,
-                     rank_count, stage_y, stage_row_bytes);
+                     make_fast_div(segments), first_rank, rank_count);
   return (int)hipGetLastError();
 }
 
 template <typename T, typename U, class CT>
-int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count,
-                     const uint8_t *stage_y, uint64_t stage_row_bytes, hipStream_t s) {
+int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint32_t rank_count, hipStream_t s) {
 #define PPLX_COMBINE(KB, VPL) \
-  return launch_combine_v<T, U, CT, KB, VPL>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s)
+  return launch_combine_v<T, U, CT, KB, VPL>(w, tab, first_rank, rank_count, s)
   // Few picks: long pieces of each row, all picks at once.  Many picks: all of them at once,
   // 1 KiB of each (eight loads per lane in flight either way) -- except for steps of a few
   // hundred to two thousand tokens, whose waves are all resident at the same moment: there the
   // picks are better taken one after the other in 7 or 8 KiB pieces by a quarter as many waves
   // (8 x 128 DSv3 tokens, top-8: 23.4 us against 25.3 us; 8 x 256: 45.8 against 46.8; from
-  // 8 x 512 on the wide form wins, 88.7 against 91.5 us, and below 8 x 64 too).  Staged rows
-  // (the K rows of a token lie side by side) stay with the wide form: 24 us against 32 us.
+  // 8 x 512 on the wide form wins, 88.7 against 91.5 us, and below 8 x 64 too).
   const uint32_t nvec_segments = (w.H / 8 + kWave - 1) / kWave;
   const uint64_t tokens = (uint64_t)rank_count * w.M;
-  if (!CT::kStaged && w.K > 4 && tokens > 384 && tokens <= 2048 && nvec_segments >= 7) {
+  if (w.K > 4 && tokens > 384 && tokens <= 2048 && nvec_segments >= 7) {
     if (nvec_segments % 7 == 0) PPLX_COMBINE(1, 7);
     PPLX_COMBINE(1, 8);
   }
@@ -217,30 +206,20 @@ int launch_combine_k(const WorldDev &w, const CT &tab, uint32_t first_rank, uint
 
 template <class CT>
 int launch_combine_t(const WorldDev &w, const CT &tab, int in_dtype, int out_dtype, hipStream_t s,
-                     uint32_t first_rank, uint32_t rank_count, const uint8_t *stage_y = nullptr,
-                     uint64_t stage_row_bytes = 0) {
+                     uint32_t first_rank, uint32_t rank_count) {
   // dtype codes follow pplx_a2a_dtype: 0 = f32, 1 = bf16, 2 = f16.
   switch (in_dtype * 4 + out_dtype) {
-    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
-    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
-    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
-    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
-    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
-    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, first_rank, rank_count, stage_y, stage_row_bytes, s);
+    case 0 * 4 + 1: return launch_combine_k<float, __bf16>(w, tab, first_rank, rank_count, s);
+    case 0 * 4 + 2: return launch_combine_k<float, _Float16>(w, tab, first_rank, rank_count, s);
+    case 1 * 4 + 1: return launch_combine_k<__bf16, __bf16>(w, tab, first_rank, rank_count, s);
+    case 1 * 4 + 2: return launch_combine_k<__bf16, _Float16>(w, tab, first_rank, rank_count, s);
+    case 2 * 4 + 1: return launch_combine_k<_Float16, __bf16>(w, tab, first_rank, rank_count, s);
+    case 2 * 4 + 2: return launch_combine_k<_Float16, _Float16>(w, tab, first_rank, rank_count, s);
     default: return (int)hipErrorInvalidValue;
   }
 }
 
 }  // namespace
-
-int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
-                              int in_dtype, int out_dtype, void *stream) {
-  if (inline_rows)
-    return launch_combine_t(w, make_inline<true>(w, inline_rows), in_dtype, out_dtype, (hipStream_t)stream, 0,
-                            w.R, sp.stage_y, sp.y_row_bytes);
-  return launch_combine_t(w, HbmCombineT<true>{w.crank}, in_dtype, out_dtype, (hipStream_t)stream, 0, w.R,
-                          sp.stage_y, sp.y_row_bytes);
-}
 
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream) {

@@ -26,20 +26,14 @@ struct HbmDispatch {
   const DispatchRank *rows;
   __device__ __forceinline__ const DispatchRank &at(uint32_t i) const { return rows[i]; }
 };
-// STAGED: combine reads the rows that combine SEND of split mode left in the world's staging
-// area instead of expert_y.
-template <bool STAGED> struct InlineCombineT {
-  static constexpr bool kStaged = STAGED;
+struct InlineCombine {
   CombineRank rows[kInlineRanks];
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
-template <bool STAGED> struct HbmCombineT {
-  static constexpr bool kStaged = STAGED;
+struct HbmCombine {
   const CombineRank *rows;
   __device__ __forceinline__ const CombineRank &at(uint32_t i) const { return rows[i]; }
 };
-typedef InlineCombineT<false> InlineCombine;
-typedef HbmCombineT<false> HbmCombine;
 
 // Pointers rebuilt from integers would be "flat" to the compiler; these casts say
 // that they are global memory, so that plain global_load / global_store are emitted.
@@ -263,9 +257,8 @@ inline InlineDispatch make_inline(const WorldDev &w, const DispatchRank *rows) {
   return t;
 }
 
-template <bool STAGED = false>
-inline InlineCombineT<STAGED> make_inline(const WorldDev &w, const CombineRank *rows) {
-  InlineCombineT<STAGED> t{};
+inline InlineCombine make_inline(const WorldDev &w, const CombineRank *rows) {
+  InlineCombine t{};
   for (uint32_t i = 0; i < w.R && i < kInlineRanks; ++i) t.rows[i] = rows[i];
   return t;
 }

@@ -134,43 +134,46 @@ struct RouteSpan {
                                   // here (and reports the faults) when set: the scatter that
                                   // follows works the slots out by itself
   uint32_t *slot_out;     // [G * M][K], indexed by absolute virtual token
-  // split mode only:
-  uint32_t *expert_out;   // [G * M][K] expert of every pair (num_experts = the pair has no row)
-  uint32_t *counts_out;   // [E] rows per expert
 };
 
-// Device state of split send / recv mode: a two-hop path through staging that the world
-// owns.  dispatch SEND routes the step and leaves one copy of the row per (token, pick) in
-// stage_x, in the order of the picks, in the reference's wire format  row | fp32 scales | u32
-// source token, padded to 16 bytes (csrc/all_to_all/intranode.cpp:41-47,
-// csrc/all_to_all/intranode_dispatch.cu:60-61,148-150); dispatch RECV moves each staged row to
-// its slot in the callers' expert-major outputs.  combine SEND copies expert rows into stage_y,
-// one row per (token, pick); combine RECV reduces them.
+// Device state of split send / recv mode: two hops through staging that the world owns.
+// The reference's SEND puts one copy of a row per pick into the inbox of the rank that owns the
+// pick's expert, because that copy has to cross a link (csrc/all_to_all/intranode_dispatch.cu:
+// 146-180); with every rank in one HBM the staging area is the wire, and one copy per TOKEN is
+// all SEND has to leave behind:
+//   dispatch SEND   copies what the call may not keep -- every present token's row, scales and
+//                   picks, and the number of tokens present in each DP group -- into stage_x /
+//                   stage_idx / stage_n (row | fp32 scales, padded to 16 bytes: the reference's
+//                   wire row, csrc/all_to_all/intranode.cpp:41-47, without the source-token tag,
+//                   which the position in the staging area stands for)
+//   dispatch RECV   is the one-call dispatch reading the staged copies and writing the outputs
+//                   named by the RECV calls
+//   combine SEND    is the one-call combine writing into stage_y, one row per (rank, token)
+//   combine RECV    copies each present token's combined row to the caller's out_tokens
 struct SplitDev {
-  uint8_t *stage_x;        // [G * M][K][token_stride]
-  uint32_t token_stride;   // round_up(Hb + 4 S + 4, 16)
+  uint8_t *stage_x;        // [G * M][token_stride]
+  uint32_t token_stride;   // round_up(Hb + 4 S, 16)
   uint32_t pad_;
-  uint32_t *gexp;          // [G * M][K] expert of a pair (num_experts = the pair has no row)
-  uint32_t *gcnt;          // [E] rows sent to expert e
-  uint8_t *stage_y;        // [G * M * K][y_row_bytes]
-  uint64_t y_row_bytes;
+  uint32_t *stage_idx;     // [G * M][K] the staged tokens' picks
+  uint32_t *stage_n;       // [G] tokens present in each DP group at SEND
+  uint8_t *stage_y;        // [R * M][H] combined rows, 2-byte elements
 };
 
-// stage_x, gexp and gcnt are one allocation, in this order, so that a kernel short of scalar
-// registers can take the first pointer alone and work out the rest.
+// stage_x, stage_idx and stage_n are one allocation, in this order.
 struct StageLayout {
   uint32_t token_stride;
-  uint64_t gexp_offset, gcnt_offset, bytes;
+  uint64_t idx_offset, n_offset, bytes;
 };
 #ifdef __HIPCC__
 __host__ __device__
 #endif
-inline StageLayout stage_layout(uint32_t row_bytes, uint32_t scales, uint64_t pairs, uint32_t experts) {
+inline StageLayout stage_layout(uint32_t row_bytes, uint32_t scales, uint64_t tokens, uint32_t picks,
+                                uint32_t groups) {
   StageLayout l;
-  l.token_stride = (row_bytes + 4u * scales + 4u + 15u) & ~15u;
-  l.gexp_offset = pairs * l.token_stride;
-  l.gcnt_offset = l.gexp_offset + pairs * 4u;
-  l.bytes = l.gcnt_offset + 4ull * experts;
+  l.token_stride = (row_bytes + 4u * scales + 15u) & ~15u;
+  l.idx_offset = tokens * l.token_stride;
+  l.n_offset = (l.idx_offset + tokens * picks * 4u + 15u) & ~15ull;
+  l.bytes = l.n_offset + ((4ull * groups + 15u) & ~15ull);
   return l;
 }
 
@@ -219,17 +222,13 @@ int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t
                     void *stream);
 int launch_combine(const WorldDev &w, const CombineRank *inline_rows, int in_dtype, int out_dtype,
                    void *stream);
-// Split mode phases, each for all ranks at once (`inline_rows` as above).  launch_split_pack is
-// the second half of a dispatch SEND whose routing ran as launches of its own.
-int launch_split_pack(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows, void *stream);
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
-                               uint32_t pick_vector, void *stream);
-int launch_split_dispatch_recv(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
-                               void *stream);
-int launch_split_combine_send(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
-                              int in_dtype, void *stream);
-int launch_split_combine_recv(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows,
-                              int in_dtype, int out_dtype, void *stream);
+// Split mode's own launches, each for all ranks at once (`inline_rows` as above): dispatch SEND
+// stages the tokens, combine RECV delivers the combined rows (`elem_bytes` of out_tokens).
+// dispatch RECV and combine SEND are launch_dispatch / launch_combine on rows that point into
+// the staging area.
+int launch_split_stage_tokens(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
+                              void *stream);
+int launch_split_deliver(const WorldDev &w, const SplitDev &sp, const CombineRank *inline_rows, void *stream);
 // True when dispatch runs as the single fused launch for this geometry.
 bool dispatch_is_fused(const WorldDev &w);
 // LDS bytes the routing kernels need for a given geometry.

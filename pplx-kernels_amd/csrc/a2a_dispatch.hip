@@ -235,14 +235,10 @@ __device__ __forceinline__ void count_earlier_picks(const WorldDev &w, const Tab
 //      lane resolves its destination row and keeps it in registers;
 //   4. the waves fan their rows out.  The last workgroup has counted everything and writes
 //      out_expert_num_tokens.
-// As dispatch SEND of split mode (`stage` = SplitDev::stage_x) the launch leaves the callers'
-// outputs alone: the row of pair (token, pick) goes to the pair's staging row, its expert and
-// the rows per expert to the tables behind the rows (stage_layout).
 template <int NV, bool EXACT, class DT>
 __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, DT tab, uint32_t ksplit,
                                                                   uint32_t kper, uint32_t tokens_per_block,
-                                                                  uint32_t pick_vector, uint32_t write_through,
-                                                                  uint8_t *stage) {
+                                                                  uint32_t pick_vector, uint32_t write_through) {
   constexpr uint32_t kFusedThreads = fused_threads(NV);
   extern __shared__ unsigned long long lds_u64[];
   Timeline timeline;
@@ -319,21 +315,7 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   Destination dst;
   if (my_in_range && lane < w.K) {
     const size_t pair = (size_t)my_v * w.K + lane;
-    if (stage != nullptr) {
-      // (whether the slot fits the receiver's rows is for RECV to say)
-      const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
-      if (my_pick_has_row) {
-        dst.row = reinterpret_cast<uint64_t>(stage + pair * lay.token_stride);
-        dst.scale = dst.row + w.Hb;
-        dst.scale_step = 1;
-        if (my_part == 0) *global_ptr<uint32_t>(dst.row + w.Hb + 4ull * w.S) = my_t;
-      }
-      if (my_part == 0) {
-        as_global(reinterpret_cast<uint32_t *>(stage + lay.gexp_offset))[pair] = my_pick_has_row ? my_e : w.E;
-      }
-    } else if (my_live) {
-      dst = resolve_destination(w, rows(), my_e, my_slot, my_part == 0);
-    }
+    if (my_live) dst = resolve_destination(w, rows(), my_e, my_slot, my_part == 0);
     if (my_live && my_part == 0) {
       as_global(w.slot_map)[pair] = my_slot;
       if (my_e >= w.E) {
@@ -346,11 +328,6 @@ __global__ __launch_bounds__(fused_threads(NV)) void dispatch_fused(WorldDev w, 
   if (blockIdx.x == gridDim.x - 1) {
     for (uint32_t e = threadIdx.x; e < w.E; e += kFusedThreads) {
       const uint32_t rows_of_e = hist[e] + __popc(own_mask[e]);
-      if (stage != nullptr) {
-        const StageLayout lay = stage_layout(w.Hb, w.S, (uint64_t)total * w.K, w.E);
-        as_global(reinterpret_cast<uint32_t *>(stage + lay.gcnt_offset))[e] = rows_of_e;
-        continue;
-      }
       const DispatchRank &owner = rows().at(owner_of(w, e));
       as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)rows_of_e;
     }
@@ -528,8 +505,7 @@ int launch_scatter_t(const WorldDev &w, const DT &tab, bool routed, hipStream_t 
 }
 
 template <class DT>
-int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s,
-                   uint8_t *stage = nullptr) {
+int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipStream_t s) {
   const uint32_t tokens = w.G * w.M;
   const uint32_t kWaves = fused_threads((int)((w.Hb / 16 + kWave - 1) / kWave)) / kWave;
   // Tokens per workgroup: as few as still give every CU a workgroup (all of a workgroup's waves
@@ -548,7 +524,7 @@ int launch_fused_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hipSt
   // Rows that fit the last-level cache with room to spare are written through into it.
   const uint64_t row_bytes = (uint64_t)tokens * w.K * (w.Hb + 4ull * w.S);
   const uint32_t write_through = row_bytes <= kWriteThroughMaxBytes ? 1u : 0u;
-#define PPLX_ROW_KERNEL_ARGS ksplit, kper, tokens_per_block, pick_vector, write_through, stage
+#define PPLX_ROW_KERNEL_ARGS ksplit, kper, tokens_per_block, pick_vector, write_through
 #define PPLX_LAUNCH_LARGE_ROW_VARIANT(KERNEL) return (int)hipErrorInvalidValue
   PPLX_DISPATCH_ROW_VARIANTS(dispatch_fused);
 #undef PPLX_LAUNCH_LARGE_ROW_VARIANT
@@ -573,7 +549,7 @@ int launch_dispatch_t(const WorldDev &w, const DT &tab, uint32_t pick_vector, hi
     span.tile_mask = reinterpret_cast<unsigned long long *>(
         reinterpret_cast<uint8_t *>(w.tile_cnt) + route_tables(w.num_tiles, w.tile_chunks, w.E).mask_offset);
   }
-  int err = launch_route_t<DT, false>(w, tab, span, s);
+  int err = launch_route_t(w, tab, span, s);
   if (err) return err;
   return launch_scatter_t(w, tab, !slots_in_scatter, s);
 }
@@ -609,34 +585,6 @@ int launch_bind_combine(const WorldDev &w, const BindCombineBatch &b, void *stre
   hipLaunchKernelGGL((bind_rows<BindCombineBatch, CombineRank>), dim3(1), dim3(256), 0,
                      (hipStream_t)stream, w.crank, b);
   return (int)hipGetLastError();
-}
-
-// dispatch SEND of split mode: the routing of the one-call form, rows into the staging area.
-template <class DT>
-int launch_split_dispatch_send_t(const WorldDev &w, const SplitDev &sp, const DT &tab, uint32_t pick_vector,
-                                 const DispatchRank *inline_rows, hipStream_t s) {
-  if (dispatch_is_fused(w)) return launch_fused_t(w, tab, pick_vector, s, sp.stage_x);
-  RouteSpan span{};
-  span.v_begin = 0;
-  span.v_count = w.G * w.M;
-  span.tile_chunks = w.tile_chunks;
-  span.pick_vector = pick_vector;
-  span.tile_cnt = w.tile_cnt;
-  span.slot_out = w.slot_map;
-  span.expert_out = sp.gexp;
-  span.counts_out = sp.gcnt;
-  int err = launch_route_t<DT, true>(w, tab, span, s);
-  if (err) return err;
-  return launch_split_pack(w, sp, inline_rows, s);
-}
-
-int launch_split_dispatch_send(const WorldDev &w, const SplitDev &sp, const DispatchRank *inline_rows,
-                               uint32_t pick_vector, void *stream) {
-  if (pick_vector != 4 && pick_vector != 2) pick_vector = 1;
-  if (inline_rows)
-    return launch_split_dispatch_send_t(w, sp, make_inline(w, inline_rows), pick_vector, inline_rows,
-                                        (hipStream_t)stream);
-  return launch_split_dispatch_send_t(w, sp, HbmDispatch{w.drank}, pick_vector, nullptr, (hipStream_t)stream);
 }
 
 int launch_dispatch(const WorldDev &w, const DispatchRank *inline_rows, uint32_t pick_vector, void *stream) {

@@ -22,11 +22,6 @@ namespace {
 // With span.tile_mask set, route_count also keeps the masks and reports the faults, and there
 // is no route_slots launch: the scatter that follows works each token's slots out of the
 // scanned counts and the masks by itself (slots_from_masks).
-//
-// SPLIT = false: the launch writes out_expert_num_tokens of the owning ranks.  SPLIT = true
-// (dispatch SEND of split mode, which may not touch the outputs yet): the rows per expert go to
-// counts_out instead, and the expert of every pair of the span (num_experts where the pair has
-// no row) to expert_out, for the later phases.
 // ---------------------------------------------------------------------------
 
 // The token of this thread: which group and sender, whether its row of picks exists, and the
@@ -130,9 +125,9 @@ __device__ __forceinline__ uint32_t slots_from_masks(const WorldDev &w, uint32_t
 
 // One wavefront per expert: tile_cnt[.][e] becomes its own exclusive prefix over the tiles, and
 // the total goes to out_expert_num_tokens of the owning rank
-// (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total) or, in split mode, to
-// counts_out.  Up to 256 tiles are fetched per trip to memory.
-template <class DT, bool SPLIT>
+// (csrc/all_to_all/intranode_dispatch.cu:221 accumulates the same total).  Up to 256 tiles are
+// fetched per trip to memory.
+template <class DT>
 __global__ __launch_bounds__(256) void route_scan(WorldDev w, DT tab, RouteSpan span, uint32_t tiles) {
   const uint32_t lane = lane_id();
   const uint32_t e = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave);
@@ -160,18 +155,14 @@ __global__ __launch_bounds__(256) void route_scan(WorldDev w, DT tab, RouteSpan 
     }
   }
   if (lane == 0) {
-    if (SPLIT) {
-      span.counts_out[e] = carry;
-    } else {
-      const DispatchRank &owner = tab.at(owner_of(w, e));
-      as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)carry;
-    }
+    const DispatchRank &owner = tab.at(owner_of(w, e));
+    as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)carry;
   }
 }
 
 // `scanned`: tile_cnt holds the rows of earlier tiles (route_scan has run); otherwise the span
 // is a single tile and this launch also writes the totals.
-template <class DT, bool SPLIT, int PV>
+template <class DT, int PV>
 __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpan span, uint32_t scanned) {
   // LDS: mask[chunks][E] (one bit per token of the chunk routed to e),
   //      then base[chunks][E] (rows of e taken before the chunk starts).
@@ -210,12 +201,8 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
       running += __popcll(lds_mask[(size_t)c * w.E + e]);
     }
     if (!scanned) {
-      if (SPLIT) {
-        span.counts_out[e] = running;
-      } else {
-        const DispatchRank &owner = tab.at(owner_of(w, e));
-        as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)running;
-      }
+      const DispatchRank &owner = tab.at(owner_of(w, e));
+      as_global(owner.out_num_tokens)[(int64_t)local_of(w, e) * owner.out_num_tokens_stride] = (int32_t)running;
     }
   }
   __syncthreads();
@@ -229,21 +216,16 @@ __global__ __launch_bounds__(1024) void route_slots(WorldDev w, DT tab, RouteSpa
         slot = lds_base[chunk * w.E + e] + __popcll(lds_mask[(size_t)chunk * w.E + e] & below);
       }
       out[k] = slot;
-      // later phases of split mode treat an id >= E as "no row"
-      if (SPLIT) span.expert_out[(size_t)tok.v * w.K + k] = slot == kInvalidSlot ? w.E : e;
       return 0u;
     });
     if (no_row.codes) atomicOr(w.faults, no_row.codes);
-  } else if (SPLIT && tok.in_span) {
-    // a token that is not there this step: none of its pairs has a row
-    for (uint32_t k = 0; k < w.K; ++k) span.expert_out[(size_t)tok.v * w.K + k] = w.E;
   }
   if (tok.in_span && tok.t == 0 && dispatch_group_overflows(w, tab, tok.g)) {
     atomicOr(w.faults, kFaultTooManyTokens);
   }
 }
 
-template <class DT, bool SPLIT, int PV>
+template <class DT, int PV>
 int launch_route_pv(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
   const uint32_t block = span.tile_chunks * kWave;
   const uint32_t tiles = (span.v_count + block - 1) / block;
@@ -251,21 +233,21 @@ int launch_route_pv(const WorldDev &w, const DT &tab, const RouteSpan &span, hip
   if (tiles > 1) {
     hipLaunchKernelGGL((route_count<DT, PV>), dim3(tiles), dim3(block),
                        span.tile_chunks * w.E * sizeof(unsigned long long), s, w, tab, span);
-    hipLaunchKernelGGL((route_scan<DT, SPLIT>), dim3((w.E + 3) / 4), dim3(256), 0, s, w, tab, span, tiles);
+    hipLaunchKernelGGL((route_scan<DT>), dim3((w.E + 3) / 4), dim3(256), 0, s, w, tab, span, tiles);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return (int)err;
     if (span.tile_mask != nullptr) return 0;  // the scatter works the slots out
   }
-  hipLaunchKernelGGL((route_slots<DT, SPLIT, PV>), dim3(tiles), dim3(block), lds, s, w, tab, span,
+  hipLaunchKernelGGL((route_slots<DT, PV>), dim3(tiles), dim3(block), lds, s, w, tab, span,
                      tiles > 1 ? 1u : 0u);
   return (int)hipGetLastError();
 }
 
-template <class DT, bool SPLIT>
+template <class DT>
 int launch_route_t(const WorldDev &w, const DT &tab, const RouteSpan &span, hipStream_t s) {
-  if (span.pick_vector == 4) return launch_route_pv<DT, SPLIT, 4>(w, tab, span, s);
-  if (span.pick_vector == 2) return launch_route_pv<DT, SPLIT, 2>(w, tab, span, s);
-  return launch_route_pv<DT, SPLIT, 1>(w, tab, span, s);
+  if (span.pick_vector == 4) return launch_route_pv<DT, 4>(w, tab, span, s);
+  if (span.pick_vector == 2) return launch_route_pv<DT, 2>(w, tab, span, s);
+  return launch_route_pv<DT, 1>(w, tab, span, s);
 }
 
 }  // namespace

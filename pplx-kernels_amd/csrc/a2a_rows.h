@@ -1,5 +1,4 @@
-// Row fan-out in registers, shared by the dispatch kernels and split mode's pack / unpack,
-// and the macro that picks the register variant for a row size.
+// Row fan-out in registers, shared by the dispatch kernels, and the macro that picks the register variant for a row size.
 #pragma once
 #include "a2a_common.h"
 

@@ -227,10 +227,10 @@ def world_of(fptr: int) -> WorldRef:
 def reserve_split(world: WorldRef, expert_y_elem_bytes: int) -> None:
     """Split send / recv calls go through staging that the library never allocates inside
     dispatch / combine.  The reference's callers do not know of it, so the operator layer
-    reserves it the first time a rank splits a call (and widens it for a wider ``expert_y``
-    dtype); like any allocation this synchronises and cannot happen under stream capture: run
-    one eager step before capturing split calls, or call this up front with the widest
-    ``expert_y`` element (a world whose split calls have been captured cannot widen any more)."""
+    reserves it the first time a rank splits a dispatch (``expert_y_elem_bytes`` 0) or a combine
+    (non-zero); like any allocation this synchronises and cannot happen under stream capture:
+    run one eager step before capturing split calls, or call this up front.  What has been
+    reserved never moves."""
     _C.reserve_split(world.fptr, expert_y_elem_bytes)
 
 

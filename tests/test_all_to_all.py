@@ -730,18 +730,21 @@ def test_split_send_recv(kw):
     for round_ in range(2):  # twice: the per-step state must reset itself
         step.expert_x_all.view(torch.uint8).fill_(0)
         step.expert_num_tokens_all.fill_(-1)
-        saved = [x.clone() for x in step.dp_x]
+        inputs = [t for seq in (step.dp_x, step.dp_x_scale, step.indices, step.bound_m) for t in seq if t is not None]
+        saved = [x.clone() for x in inputs]
         for r in range(R):
             ranks[r].dispatch(**_dispatch_kw(step, r), do_send=True, do_recv=False)
-        # SEND has consumed the inputs and must not have touched the outputs yet
+        # SEND has consumed the inputs (rows, scales, picks and token counts: the caller may
+        # reuse all of them) and must not have touched the outputs yet
         torch.cuda.synchronize()
         assert int(step.expert_x_all.view(torch.uint8).max()) == 0
         assert int(step.expert_num_tokens_all.max()) == -1
-        for x in step.dp_x:
+        for x in inputs:
             x.view(torch.uint8).fill_(0x7F)
         for r in reversed(range(R)):
             ranks[r].dispatch(**_dispatch_kw(step, r), do_send=False, do_recv=True)
-        for x, s_ in zip(step.dp_x, saved):
+        torch.cuda.synchronize()
+        for x, s_ in zip(inputs, saved):
             x.copy_(s_)
         expected = check_dispatch_against_oracle(step)
 
