@@ -718,6 +718,11 @@ def _combine_kw(step, r):
         dict(name="split-f32y", expert_y_dtype=torch.float32, out_dtype=torch.float16),
         # a step of a few hundred tokens, top-6: combine RECV takes its picks one at a time
         dict(name="split-mid", max_num_tokens=128, experts_per_token=6, hidden_dim=7168),
+        # worlds whose rank tables live in HBM: the rows that point into the staging area are bound like any others
+        dict(name="split-72-ranks", world_size=72, num_experts=144, experts_per_token=4, max_num_tokens=5,
+             hidden_dim=512, in_dtype=FP8),
+        dict(name="split-80-ranks-dp2", world_size=80, dp_size=2, num_experts=160, experts_per_token=8,
+             max_num_tokens=70, hidden_dim=1024),
     ],
     ids=lambda kw: kw["name"],
 )
