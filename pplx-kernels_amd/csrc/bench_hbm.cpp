@@ -10,6 +10,10 @@
 //   streams    the same 2 GiB written (read) in 4 KiB pieces that go round-robin to S regions of
 //              the buffer: S = 256 is what a dispatch into 256 experts' buffers does to the
 //              memory, S = 8 what a dispatch into 8 experts' buffers does
+//   rows       2 GiB written as rows of 4, 7 or 8 KiB, one wavefront (a workgroup of its own) per
+//              row, the rows in address order or scattered over the buffer one by one: what the
+//              shape of the scatter (one wave, one row, 16 bytes per lane and store) gets from
+//              the memory whatever it is asked to route
 //
 // Every kernel moves 16 bytes per lane and access, eight accesses in flight per lane, with
 // non-temporal stores; buffers are 2 GiB, far beyond the 256 MB last-level cache.  Times are
@@ -147,6 +151,31 @@ __global__ __launch_bounds__(kThreads) void read_streams_kernel(const u32x4 *src
   if (x[0] == 0xdeadbeefu && x[1] == 0x12345678u) *sink = x;
 }
 
+// One wavefront per row of `row_vectors` 16-byte vectors (NV per lane); row r goes to position
+// (r * mult) % rows: mult = 1 writes in address order, a mult coprime to `rows` scatters.
+template <int NV>
+__global__ __launch_bounds__(64) void write_rows_kernel(u32x4 *dst, uint32_t rows, uint32_t row_vectors, uint32_t mult) {
+  const uint32_t lane = threadIdx.x;
+  const uint32_t row = blockIdx.x;
+  if (row >= rows) return;
+  const uint32_t place = (uint32_t)(((uint64_t)row * mult) % rows);
+  u32x4 *out = dst + (uint64_t)place * row_vectors;
+  const u32x4 v = {lane, row, 3u, 4u};
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (lane + i * 64u < row_vectors) __builtin_nontemporal_store(v, out + lane + i * 64u);
+  }
+}
+
+uint32_t gcd(uint32_t a, uint32_t b) {
+  while (b) {
+    const uint32_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a;
+}
+
 template <class Launch>
 void measure(const char *name, double bytes, unsigned repeats, hipStream_t stream, Launch &&launch) {
   hipEvent_t a, b;
@@ -235,6 +264,22 @@ int main(int argc, char **argv) {
       snprintf(name, sizeof name, "read: 4 KiB pieces out of %u regions in turn", streams);
       measure(name, (double)big, repeats, stream, [&] {
         hipLaunchKernelGGL(read_streams_kernel, dim3(pieces), block, 0, stream, a, streams, spacing, sink);
+      });
+    }
+  }
+  for (uint32_t row_vectors : {256u, 448u, 512u}) {
+    const uint32_t rows = (uint32_t)(big_vectors / row_vectors);
+    for (bool scattered : {false, true}) {
+      uint32_t mult = 1;
+      if (scattered) {
+        mult = (uint32_t)(rows * 0.6180339887) | 1u;
+        while (gcd(mult, rows) != 1) mult += 2;
+      }
+      char name[96];
+      snprintf(name, sizeof name, "rows: %u KiB rows, one wave each, %s", row_vectors / 64,
+               scattered ? "scattered" : "in address order");
+      measure(name, (double)rows * row_vectors * 16.0, repeats, stream, [&] {
+        hipLaunchKernelGGL(write_rows_kernel<8>, dim3(rows), dim3(64), 0, stream, b, rows, row_vectors, mult);
       });
     }
   }
