@@ -718,6 +718,8 @@ def _combine_kw(step, r):
         dict(name="split-f32y", expert_y_dtype=torch.float32, out_dtype=torch.float16),
         # a step of a few hundred tokens, top-6: combine RECV takes its picks one at a time
         dict(name="split-mid", max_num_tokens=128, experts_per_token=6, hidden_dim=7168),
+        # no bound_m: the token counts that SEND stages are the tensors' row counts
+        dict(name="split-no-bound-m", tokens="max", no_bound_m=True, in_dtype=FP8, hidden_dim=512),
         # worlds whose rank tables live in HBM: the rows that point into the staging area are bound like any others
         dict(name="split-72-ranks", world_size=72, num_experts=144, experts_per_token=4, max_num_tokens=5,
              hidden_dim=512, in_dtype=FP8),
@@ -727,9 +729,11 @@ def _combine_kw(step, r):
     ids=lambda kw: kw["name"],
 )
 def test_split_send_recv(kw):
+    kw = dict(kw)
+    with_bound_m = not kw.pop("no_bound_m", False)
     spec = _small_spec(**kw)
     groups = generate(spec)
-    step = DeviceStep(spec, groups)
+    step = DeviceStep(spec, groups, with_bound_m=with_bound_m)
     ranks = _make_ranks(spec, kw["name"])
     R = spec.world_size
     for round_ in range(2):  # twice: the per-step state must reset itself
