@@ -27,7 +27,8 @@ dominated by a thread that has just woken up (see ``wake_host``).
 
 The decode shape C3 additionally carries ``graph_replay_1000x_us``: ONE captured graph over ONE
 buffer set replayed 1000 times, the form its specification names; 12.5 MB replayed back to back
-stay in the last-level cache, so that figure is cache-resident and carries no HBM fraction.
+stay in the last-level cache, so that figure is cache-resident and carries no HBM fraction;
+``bound_eager_1000x_us`` is the same thousand steps on that one buffer set as eager launches.
 ``roofline`` is for the dominant kernel of the headline workload (``combine_gather``):
 algorithmic bytes per launch divided by its mean duration, measured with HIP events around graph
 replays that contain only launches of that kernel; ``traffic`` is read from the rocprofv3 counter
@@ -231,10 +232,14 @@ def measure_workload(name, spec, steps_k, warmup):
 
     graphs = [capture(world, stream, both(st)) for st in steps]
     graph_us = time_graphs(graphs, order, stream, warmup)
-    replay_1000 = None
+    replay_1000 = eager_1000 = None
     if name == "C3":
-        # the form the decode shape is specified in: ONE graph, replayed 1000 times back to back
+        # the form the decode shape is specified in: ONE graph, replayed 1000 times back to back ...
         replay_1000 = time_graphs([graphs[0]], [0], stream, warmup, GRAPH_REPLAYS_C3)
+        # ... and the same 1000 steps on that one buffer set as eager launches of the bound step
+        eager_1000 = time_steps(
+            lambda i: (bound[0].dispatch(stream), bound[0].combine(stream)), [0] * GRAPH_REPLAYS_C3, stream, warmup
+        )
     for g in graphs:
         g.destroy()
     del bound
@@ -277,6 +282,7 @@ def measure_workload(name, spec, steps_k, warmup):
     }
     if replay_1000 is not None:
         out["graph_replay_1000x_us"] = replay_1000
+        out["bound_eager_1000x_us"] = eager_1000
         out["graph_replay_1000x_note"] = (
             f"one hipGraph over one buffer set replayed {GRAPH_REPLAYS_C3} times back to back: the "
             f"{(disp_b + comb_b) / 1e6:.1f} MB of a step stay in the 256 MB last-level cache, so this is a "
@@ -491,7 +497,7 @@ def steps_for(name, steps_k):
 COMPACT_FIELDS = (
     "workload", "tokens", "pairs", "buffer_sets", "steps_timed", "launch_form", "step_us", "step_us_regions",
     "bound_eager_step_us", "bound_eager_host_us_per_call", "graph_step_us", "per_rank_api_step_us", "per_rank_api_calls_per_step", "dispatch_us",
-    "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac", "graph_replay_1000x_us",
+    "combine_us", "step_hbm_frac", "dispatch_hbm_frac", "combine_hbm_frac", "graph_replay_1000x_us", "bound_eager_1000x_us",
     "graph_replay_1000x_note",
 )  # fmt: skip
 
