@@ -28,6 +28,11 @@ import torch
 from . import ops
 from .ops import _C, _ops
 
+# (bound once: a step of R simulated ranks makes 2 R of these calls)
+_is_compiling = torch.compiler.is_compiling
+_eager_dispatch = _C.dispatch
+_eager_combine = _C.combine
+
 
 class AllToAll:
     def __init__(
@@ -81,7 +86,7 @@ class AllToAll:
         # Under torch.compile the call goes through the registered op (what the reference always
         # does, src/pplx_kernels/all_to_all.py:47-59) so that it traces; an eager call enters the
         # op's implementation directly, without the dispatcher's boxing of ten arguments.
-        fn = self._dispatch_fn if torch.compiler.is_compiling() else _C.dispatch
+        fn = self._dispatch_fn if _is_compiling() else _eager_dispatch
         fn(
             self._ptr,
             out_expert_num_tokens,
@@ -108,7 +113,7 @@ class AllToAll:
         """``out_tokens[t] = sum_k weights[t, k] * expert_y[slot of (t, k)]`` for
         ``t < bound_m``, fp32 accumulation in pick order; later rows are left as they are."""
         assert self._ptr is not None
-        fn = self._combine_fn if torch.compiler.is_compiling() else _C.combine
+        fn = self._combine_fn if _is_compiling() else _eager_combine
         fn(
             self._ptr,
             out_tokens,
